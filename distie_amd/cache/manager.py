@@ -31,7 +31,7 @@ from typing import Dict, Hashable, List, Optional, Sequence
 
 import torch
 
-from ..parts.base import FixedState, PagedTensors
+from ..parts.base import Borrowed, CacheNeeds, FixedState, PagedTensors
 from .block_pool import BlockPool, OutOfBlocks
 
 GONE = -1
@@ -115,29 +115,28 @@ class CacheManager:
         self._layers: List[LayerCache] = []
         self._state_slabs: List[torch.Tensor] = []
         by_need: Dict[PagedTensors, CacheGroup] = {}
+        borrowers: List[tuple] = []
         for layer, needs in enumerate(requirements):
             if not isinstance(needs, dict):
                 needs = {"mixer": needs}
             views = LayerCache()
             self._layers.append(views)
             for name, need in needs.items():
-                if isinstance(need, PagedTensors):
-                    if need not in by_need:
-                        by_need[need] = CacheGroup(need, [], BlockPool(self.num_blocks))
-                        self.groups.append(by_need[need])
-                    by_need[need].members.append((layer, name))
-                elif isinstance(need, FixedState):
-                    slabs = {}
-                    for decl in need.tensors:
+                paged, state = self._split(need, layer, name)
+                view = views.views[name] = CacheView()
+                if isinstance(paged, PagedTensors):
+                    if paged not in by_need:
+                        by_need[paged] = CacheGroup(paged, [], BlockPool(self.num_blocks))
+                        self.groups.append(by_need[paged])
+                    by_need[paged].members.append((layer, name))
+                elif isinstance(paged, Borrowed):
+                    borrowers.append((layer, name, paged))
+                if state is not None:
+                    for decl in state.tensors:
                         if allocate:
-                            slabs[decl.name] = torch.zeros((self.num_slots + 1, *decl.shape),
-                                                           dtype=decl.dtype or torch.float32, device=device)
-                            self._state_slabs.append(slabs[decl.name])
-                    views.views[name] = CacheView(tensors=slabs)
-                elif need is None:
-                    views.views[name] = CacheView()
-                else:
-                    raise TypeError(f"layer {layer}, {name}: unknown cache requirement {need!r}")
+                            view.tensors[decl.name] = torch.zeros((self.num_slots + 1, *decl.shape),
+                                                                  dtype=decl.dtype or torch.float32, device=device)
+                            self._state_slabs.append(view.tensors[decl.name])
         for index, group in enumerate(self.groups):
             need = group.requirement
             if allocate:
@@ -145,11 +144,36 @@ class CacheManager:
                     shape = (len(group.members), self.num_blocks + 1) + need.page_shape(decl, self.block_size)
                     group.tensors[decl.name] = torch.zeros(shape, dtype=decl.dtype or dtype, device=device)
             for i, (layer, name) in enumerate(group.members):
-                self._layers[layer].views[name] = CacheView(
-                    group=index, tensors={n: slab[i] for n, slab in group.tensors.items()})
+                view = self._layers[layer].views[name]
+                view.group = index
+                view.tensors.update({n: slab[i] for n, slab in group.tensors.items()})
+        members = {member: group for group in self.groups for member in group.members}
+        for layer, name, source in borrowers:
+            lender = (source.layer, source.name)
+            if lender not in members or lender == (layer, name):
+                raise ValueError(f"layer {layer}, {name}: borrows the pages of layer {source.layer}, {source.name}, "
+                                 f"which keeps none")
+            view, lent = self._layers[layer].views[name], self._layers[source.layer].views[source.name]
+            view.group = lent.group
+            view.tensors.update({decl.name: lent.tensors[decl.name] for decl in members[lender].requirement.tensors
+                                 if decl.name in lent.tensors})
         self.slots = BlockPool(self.num_slots)
         self._requests: Dict[Hashable, RequestCache] = {}
         self.table_width = 0
+
+    @staticmethod
+    def _split(need, layer=None, name=None):
+        """-> (PagedTensors | Borrowed | None, FixedState | None) of one declaration."""
+        if isinstance(need, CacheNeeds):
+            paged, state = need.paged, need.state
+        elif isinstance(need, FixedState):
+            paged, state = None, need
+        else:
+            paged, state = need, None
+        if paged is not None and not isinstance(paged, (PagedTensors, Borrowed)) or \
+                state is not None and not isinstance(state, FixedState):
+            raise TypeError(f"layer {layer}, {name}: unknown cache requirement {need!r}")
+        return paged, state
 
     @staticmethod
     def page_bytes(requirements: Sequence, block_size: int, dtype=torch.float32) -> int:
@@ -158,6 +182,7 @@ class CacheManager:
         total = 0
         for needs in requirements:
             for need in (needs.values() if isinstance(needs, dict) else [needs]):
+                need = CacheManager._split(need)[0]
                 if isinstance(need, PagedTensors):
                     for decl in need.tensors:
                         count = 1

@@ -11,6 +11,7 @@ from __future__ import annotations
 from typing import Any, Dict, Mapping
 
 from .model_config import ConfigError, ModelSpec, Qwen2Config, read_config_json
+from .musutar_config import MusutarConfig
 
 _ARCHITECTURES: Dict[str, Any] = {}
 
@@ -28,6 +29,8 @@ def known_architectures() -> list:
 
 def architecture_of(config_json: Mapping[str, Any]) -> str:
     names = config_json.get("architectures")
+    if not names and isinstance(config_json.get("architecture"), str):
+        names = [config_json["architecture"]]          # some designs name theirs in the singular
     if not names or not isinstance(names, (list, tuple)):
         raise ConfigError("config.json lacks 'architectures'; known: " + ", ".join(known_architectures()))
     name = str(names[0])
@@ -50,3 +53,4 @@ def model_spec_from_dir(model_dir) -> ModelSpec:
 
 
 register_architecture(Qwen2Config.architecture, Qwen2Config)
+register_architecture(MusutarConfig.architecture, MusutarConfig)

@@ -1,0 +1,474 @@
+// Kernels of mixers and arrangements that carry something from token to token besides keys and values:
+// several residual streams with learned read, mix and write weights; a short causal convolution over time
+// whose last inputs are a request's state; attention projections with such a convolution, a partial rotation
+// and the cache write behind it; a decayed outer-product state (linear attention) scanned over the tokens;
+// gates. Everything the card of such a design wants in 32-bit is float32 here in either precision: the
+// streams, norm statistics, angles, the state and every sum that enters it.
+//
+// A step is a flattened batch: token t belongs to request token_request[t], whose new tokens are rows
+// cu_q[b] .. cu_q[b+1]-1 and whose state is row state_slots[b] of a state tensor.
+#include "common.h"
+
+namespace {
+
+constexpr int MAX_STREAMS = 8;
+constexpr int MAX_TAPS = 16;
+
+__device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + __expf(-x)); }
+__device__ __forceinline__ float siluf(float x) { return x / (1.f + __expf(-x)); }
+
+// ---------------------------------------------------------------------------------------------------
+// Residual streams. streams float32 [T, S, C]. In this order, each step optional:
+//   init:   x_s = init[t] for every s                                   (the embedding output)
+//   write:  x_j <- sum_s mix[s, j] x_s + out_w[j] * y * sigmoid(gate)   (all streams at once from the old ones)
+//   read:   u = sum_s in_w[s] x_s;  h = norm(u) * weight                (kind 0: u itself, 1: centred, 2: root mean square)
+// One block a token; u of the whole row waits in LDS between the two passes of the statistics.
+template <typename Y, typename G, typename W, typename H>
+__global__ void hyper_step_kernel(float* __restrict__ streams, int S, const float* __restrict__ init, const Y* __restrict__ y,
+                                  int y_slices, int64_t y_slice_stride, const G* __restrict__ gate, int64_t gate_ld,
+                                  const float* __restrict__ mix, const float* __restrict__ out_w,
+                                  const float* __restrict__ in_w, const W* __restrict__ norm_w, int kind, float eps,
+                                  H* __restrict__ h, int C) {
+  extern __shared__ float row[];
+  __shared__ float scratch[16];
+  const int64_t t = blockIdx.x;
+  float* x = streams + t * S * C;
+  float m[MAX_STREAMS * MAX_STREAMS], ow[MAX_STREAMS], iw[MAX_STREAMS];
+  if (y != nullptr) {
+    for (int i = 0; i < S * S; ++i) m[i] = mix[i];
+    for (int i = 0; i < S; ++i) ow[i] = out_w[i];
+  }
+  if (h != nullptr)
+    for (int i = 0; i < S; ++i) iw[i] = in_w[i];
+  float sum = 0.f;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float v[MAX_STREAMS];
+    if (init != nullptr) {
+      const float e = init[t * C + c];
+      for (int s = 0; s < S; ++s) v[s] = e;
+    } else {
+      for (int s = 0; s < S; ++s) v[s] = x[s * C + c];
+    }
+    if (y != nullptr) {
+      float d = sum_strided(y + t * C + c, y_slices, y_slice_stride);
+      if (gate != nullptr) d *= sigmoidf(to_float(gate[t * gate_ld + c]));
+      float n[MAX_STREAMS];
+      for (int j = 0; j < S; ++j) {
+        float a = 0.f;
+        for (int s = 0; s < S; ++s) a += m[s * S + j] * v[s];
+        n[j] = a + ow[j] * d;
+      }
+      for (int j = 0; j < S; ++j) v[j] = n[j];
+    }
+    if (init != nullptr || y != nullptr)
+      for (int s = 0; s < S; ++s) x[s * C + c] = v[s];
+    if (h != nullptr) {
+      float u = 0.f;
+      for (int s = 0; s < S; ++s) u += iw[s] * v[s];
+      row[c] = u;
+      sum += kind == 2 ? u * u : u;
+    }
+  }
+  if (h == nullptr) return;
+  H* out = h + t * C;
+  if (kind == 0) {
+    for (int c = threadIdx.x; c < C; c += blockDim.x) out[c] = from_float<H>(row[c]);
+    return;
+  }
+  sum = block_sum(sum, scratch);
+  float mean = 0.f, scale;
+  if (kind == 1) {
+    mean = sum / C;
+    float dev = 0.f;
+    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+      const float d = row[c] - mean;
+      dev += d * d;
+    }
+    dev = block_sum(dev, scratch);
+    scale = 1.f / sqrtf(dev / C + eps);
+  } else {
+    scale = 1.f / sqrtf(sum / C + eps);
+  }
+  for (int c = threadIdx.x; c < C; c += blockDim.x)
+    out[c] = from_float<H>((row[c] - mean) * scale * to_float(norm_w[c]));
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Short causal convolution over time, one filter a channel:
+//   out[t, c] = (residual ? x[t, c] : 0) + sum_j w[c, j] * x_(t - taps + 1 + j)[c],
+// inputs before the start of the step's rows come from the request's state (float32 [slots, taps - 1, N], the
+// last taps - 1 inputs, oldest first; zeros at the start of a sequence). A request that brings one token has
+// its state moved on here as well (nobody else reads it); the others by `conv_state_kernel` behind this one.
+template <typename X>
+__device__ __forceinline__ float conv_at(const X* __restrict__ x, int64_t ldx, const float* __restrict__ state,
+                                         const float* w, int taps, int64_t t, int i, int c, int N) {
+  float acc = 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int back = taps - 1 - j;                       // how many tokens before t
+    const float v = back <= i ? to_float(x[(t - back) * ldx + c]) : state[static_cast<int64_t>(taps - 1 - (back - i)) * N + c];
+    acc += w[j] * v;
+  }
+  return acc;
+}
+
+template <typename X, typename W, typename O>
+__global__ void causal_conv_kernel(const X* __restrict__ x, int64_t ldx, const W* __restrict__ weight, int taps,
+                                   float* __restrict__ state, O* __restrict__ out, int64_t ldo, int residual,
+                                   const int32_t* __restrict__ cu_q, const int32_t* __restrict__ token_request,
+                                   const int32_t* __restrict__ state_slots, int N) {
+  const int64_t t = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= N) return;
+  const int b = token_request[t];
+  const int first = cu_q[b];
+  const int i = static_cast<int>(t) - first;
+  const int n = cu_q[b + 1] - first;
+  float* own = state + static_cast<int64_t>(state_slots[b]) * (taps - 1) * N;
+  float w[MAX_TAPS];
+  for (int j = 0; j < taps; ++j) w[j] = to_float(weight[static_cast<int64_t>(c) * taps + j]);
+  float acc = conv_at(x, ldx, own, w, taps, t, i, c, N);
+  const float self = to_float(x[t * ldx + c]);
+  if (residual) acc += self;
+  out[t * ldo + c] = from_float<O>(acc);
+  if (n == 1) {
+    float keep[MAX_TAPS];
+    for (int k = 1; k < taps - 1; ++k) keep[k] = own[static_cast<int64_t>(k) * N + c];
+    for (int k = 1; k < taps - 1; ++k) own[static_cast<int64_t>(k - 1) * N + c] = keep[k];
+    if (taps > 1) own[static_cast<int64_t>(taps - 2) * N + c] = self;
+  }
+}
+
+// new state = the last taps - 1 of (old state, the step's rows), for requests that bring `skip_single ? > 1 : >= 1` rows
+template <typename X>
+__global__ void conv_state_kernel(const X* __restrict__ x, int64_t ldx, int taps, float* __restrict__ state,
+                                  const int32_t* __restrict__ cu_q, const int32_t* __restrict__ state_slots, int N,
+                                  int skip_single) {
+  const int b = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= N) return;
+  const int first = cu_q[b];
+  const int n = cu_q[b + 1] - first;
+  if (n < 1 || (n == 1 && skip_single)) return;
+  float* own = state + static_cast<int64_t>(state_slots[b]) * (taps - 1) * N;
+  float keep[MAX_TAPS];
+  for (int k = 0; k < taps - 1; ++k) {
+    const int s = n + k - (taps - 1);                    // row of the step, or behind its start
+    keep[k] = s >= 0 ? to_float(x[static_cast<int64_t>(first + s) * ldx + c]) : own[static_cast<int64_t>(n + k) * N + c];
+  }
+  for (int k = 0; k < taps - 1; ++k) own[static_cast<int64_t>(k) * N + c] = keep[k];
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Behind the stacked projection of attention: product [T, ld] holds q (H heads of D), then k (G heads of D) and
+// v (G heads of E) unless `has_kv` is 0. Each channel goes through its short convolution (taps 0: none); the
+// first 2 * pairs dimensions of every q and k head are turned by the token's angle (pair (j, j + pairs); cosine
+// and sine from `table` [T, pairs, 2], both times `magnitude`); q goes to q_out [T, H, DP] (zeros beyond D), k
+// and v to the token's slot of the cache, k [pages, G, P, DP], v [pages, G, DP, P] (what lies beyond D and E there
+// was zero when the cache was made and is never written).
+template <typename X, typename W, typename Q, typename C>
+__global__ void conv_rope_kv_write_kernel(const X* __restrict__ product, int64_t ld, const W* __restrict__ weight, int taps,
+                                          const float* __restrict__ state, const float2* __restrict__ table, int pairs,
+                                          float magnitude, Q* __restrict__ q_out, C* __restrict__ k_cache,
+                                          C* __restrict__ v_cache, const int32_t* __restrict__ slots,
+                                          const int32_t* __restrict__ cu_q, const int32_t* __restrict__ token_request,
+                                          const int32_t* __restrict__ state_slots, int H, int G, int D, int E, int DP,
+                                          int block_size, int has_kv, int write) {
+  const int64_t t = blockIdx.x;
+  const int N = H * D + (has_kv ? G * (D + E) : 0);
+  const int b = token_request[t];
+  const int i = static_cast<int>(t) - cu_q[b];
+  const float* own = taps > 1 ? state + static_cast<int64_t>(state_slots[b]) * (taps - 1) * N : nullptr;
+  const int64_t slot = (has_kv && write) ? slots[t] : 0;
+  const int64_t page = slot / block_size;
+  const int offset = static_cast<int>(slot % block_size);
+  auto value = [&](int c) {
+    if (taps < 1) return to_float(product[t * ld + c]);
+    float w[MAX_TAPS];
+    for (int j = 0; j < taps; ++j) w[j] = to_float(weight[static_cast<int64_t>(c) * taps + j]);
+    return conv_at(product, ld, own, w, taps, t, i, c, N);
+  };
+  // q and k: a thread owns a pair, or a single dimension beyond the turned ones; (H + G) heads of DP places
+  const int turned = has_kv ? H + G : H;
+  const int per_head = DP - pairs;                       // pairs count once
+  for (int item = threadIdx.x; item < turned * per_head; item += blockDim.x) {
+    const int head = item / per_head;
+    const int j = item % per_head;
+    const int base = head * D;                           // q heads, then k heads: both D wide, one after the other
+    float a, bq = 0.f;
+    int d0, d1 = -1;
+    if (j < pairs) {
+      d0 = j;
+      d1 = j + pairs;
+      const float x0 = value(base + d0), x1 = value(base + d1);
+      const float2 e = table[t * pairs + j];
+      const float cs = e.x * magnitude, sn = e.y * magnitude;
+      a = x0 * cs - x1 * sn;
+      bq = x1 * cs + x0 * sn;
+    } else {
+      d0 = j + pairs;
+      a = d0 < D ? value(base + d0) : 0.f;
+    }
+    if (head < H) {
+      Q* q = q_out + (t * H + head) * DP;
+      q[d0] = from_float<Q>(a);
+      if (d1 >= 0) q[d1] = from_float<Q>(bq);
+    } else if (write && d0 < D) {
+      C* k = k_cache + ((page * G + (head - H)) * block_size + offset) * DP;
+      k[d0] = from_float<C>(to_float(from_float<Q>(a)));
+      if (d1 >= 0) k[d1] = from_float<C>(to_float(from_float<Q>(bq)));
+    }
+  }
+  if (!has_kv || !write) return;
+  for (int item = threadIdx.x; item < G * E; item += blockDim.x) {
+    const int head = item / E;
+    const int e = item % E;
+    const float v = value((H + G) * D + item);
+    v_cache[((page * G + head) * DP + e) * block_size + offset] = from_float<C>(to_float(from_float<Q>(v)));
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// out[t, h * E + e] = x[t, h * ldh + e] * sigmoid(gates[t, ldg-row][h * E + e])
+template <typename X, typename G, typename O>
+__global__ void sigmoid_gate_kernel(const X* __restrict__ x, int ldh, int E, const G* __restrict__ gates, int64_t ldg,
+                                    O* __restrict__ out, int width) {
+  const int64_t t = blockIdx.x;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
+    const int head = c / E, e = c % E;
+    const float v = to_float(x[(t * (width / E) + head) * ldh + e]);
+    out[t * width + c] = from_float<O>(v * sigmoidf(to_float(gates[t * ldg + c])));
+  }
+}
+
+// out = x / sqrt(mean(x^2) + eps) * weight * sigmoid(gate): the norm over all heads together, then the gate
+template <typename W, typename G, typename O>
+__global__ void rmsnorm_gate_kernel(const float* __restrict__ x, const W* __restrict__ weight, float eps,
+                                    const G* __restrict__ gates, int64_t ldg, O* __restrict__ out, int N) {
+  __shared__ float scratch[16];
+  const int64_t t = blockIdx.x;
+  const float* row = x + t * N;
+  float sq = 0.f;
+  for (int c = threadIdx.x; c < N; c += blockDim.x) sq += row[c] * row[c];
+  sq = block_sum(sq, scratch);
+  const float scale = 1.f / sqrtf(sq / N + eps);
+  for (int c = threadIdx.x; c < N; c += blockDim.x) {
+    float v = row[c] * scale * to_float(weight[c]);
+    if (gates != nullptr) v *= sigmoidf(to_float(gates[t * ldg + c]));
+    out[t * N + c] = from_float<O>(v);
+  }
+}
+
+// kinds: 0 relu squared, 1 silu, 2 gelu (tanh form), 3 relu
+template <typename T>
+__global__ void activation_kernel(const T* __restrict__ in, int slices, int64_t slice_stride, T* __restrict__ out,
+                                  int64_t count, int kind) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  const float z = slices == 1 ? to_float(in[i]) : 0.f;
+  float r;
+  if (kind == 0) {
+    const float p = fmaxf(z, 0.f);
+    r = p * p;
+  } else if (kind == 1) {
+    r = siluf(z);
+  } else if (kind == 2) {
+    r = 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  } else {
+    r = fmaxf(z, 0.f);
+  }
+  out[i] = from_float<T>(r);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Decayed outer-product state, token by token:  S <- decay_h S + k v^T,  o = S^T q  per head, with
+// q = silu(product q), k = silu(product k), v = silu(product v); product [T, ld] holds q (H x D), k (H x D),
+// v (H x E). state float32 [slots, H, D, E]. A block owns 64 columns e of one head of one request and walks the
+// request's rows in order; thread (e, part) keeps rows d = part, part + PARTS, ... of its column in registers,
+// the PARTS partial sums of a column meet in LDS.
+template <typename X, int PARTS, int ROWS>
+__global__ void __launch_bounds__(64 * PARTS)
+decay_scan_kernel(const X* __restrict__ product, int64_t ld, float* __restrict__ state, const float* __restrict__ decay,
+                  float* __restrict__ out, const int32_t* __restrict__ cu_q, const int32_t* __restrict__ state_slots,
+                  int H, int D, int E) {
+  __shared__ float q_s[PARTS * ROWS], k_s[PARTS * ROWS];
+  __shared__ float partial[PARTS][64];
+  const int b = blockIdx.x, head = blockIdx.y;
+  const int lane = threadIdx.x % 64, part = threadIdx.x / 64;
+  const int e = blockIdx.z * 64 + lane;
+  const int first = cu_q[b], last = cu_q[b + 1];
+  const float rate = decay[head];
+  float* own = state + (static_cast<int64_t>(state_slots[b]) * H + head) * D * E;
+  float s[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    const int d = part + r * PARTS;
+    s[r] = (d < D && e < E) ? own[static_cast<int64_t>(d) * E + e] : 0.f;
+  }
+  for (int t = first; t < last; ++t) {
+    const X* row = product + static_cast<int64_t>(t) * ld;
+    __syncthreads();
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+      q_s[d] = siluf(to_float(row[head * D + d]));
+      k_s[d] = siluf(to_float(row[(H + head) * D + d]));
+    }
+    const float v = e < E ? siluf(to_float(row[2 * H * D + head * E + e])) : 0.f;
+    __syncthreads();
+    float o = 0.f;
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      const int d = part + r * PARTS;
+      if (d < D) {
+        s[r] = rate * s[r] + k_s[d] * v;
+        o += s[r] * q_s[d];
+      }
+    }
+    partial[part][lane] = o;
+    __syncthreads();
+    if (part == 0 && e < E) {
+      float total = 0.f;
+#pragma unroll
+      for (int p = 0; p < PARTS; ++p) total += partial[p][lane];
+      out[(static_cast<int64_t>(t) * H + head) * E + e] = total;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    const int d = part + r * PARTS;
+    if (d < D && e < E) own[static_cast<int64_t>(d) * E + e] = s[r];
+  }
+}
+
+}  // namespace
+
+extern "C" int distie_hyper_step(float* streams, int S, const float* init, const void* y, int y_dtype, int y_slices,
+                                 const void* gate, int gate_dtype, int64_t gate_ld, const float* mix, const float* out_w,
+                                 const float* in_w, const void* norm_w, int norm_dtype, int kind, float eps, void* h,
+                                 int h_dtype, int T, int C, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (S < 1 || S > MAX_STREAMS || C < 1 || kind < 0 || kind > 2 || y_slices < 1) return DISTIE_BAD_ARGUMENT;
+  if (y != nullptr && (mix == nullptr || out_w == nullptr)) return DISTIE_BAD_ARGUMENT;
+  if (h != nullptr && (in_w == nullptr || (kind != 0 && norm_w == nullptr))) return DISTIE_BAD_ARGUMENT;
+  if (static_cast<size_t>(C) * sizeof(float) > 64 * 1024) return DISTIE_BAD_ARGUMENT;
+  const int threads = C >= 2048 ? 512 : (C >= 512 ? 256 : (C >= 128 ? 128 : 64));
+  const size_t lds = h != nullptr ? static_cast<size_t>(C) * sizeof(float) : 0;
+  const int64_t y_stride = static_cast<int64_t>(T) * C;
+  if (y == nullptr) y_dtype = DISTIE_F32;
+  if (gate == nullptr) gate_dtype = y_dtype;
+  if (norm_w == nullptr) norm_dtype = DISTIE_F32;
+  if (h == nullptr) h_dtype = DISTIE_F32;
+  DISTIE_DISPATCH(y_dtype, Y, DISTIE_DISPATCH(gate_dtype, G, DISTIE_DISPATCH(norm_dtype, W, DISTIE_DISPATCH(h_dtype, HT,
+      hyper_step_kernel<Y, G, W, HT><<<T, threads, lds, stream>>>(
+          streams, S, init, static_cast<const Y*>(y), y_slices, y_stride, static_cast<const G*>(gate), gate_ld, mix, out_w,
+          in_w, static_cast<const W*>(norm_w), kind, eps, static_cast<HT*>(h), C)))));
+  return launch_status();
+}
+
+extern "C" int distie_causal_conv(const void* x, int x_dtype, int64_t ldx, const void* weight, int w_dtype, int taps,
+                                  float* state, void* out, int out_dtype, int64_t ldo, int residual, const int32_t* cu_q,
+                                  const int32_t* token_request, const int32_t* state_slots, int T, int N,
+                                  hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (taps < 1 || taps > MAX_TAPS || N < 1 || ldx < N || ldo < N || (taps > 1 && state == nullptr)) return DISTIE_BAD_ARGUMENT;
+  const int threads = N >= 256 ? 256 : (N >= 128 ? 128 : 64);
+  const dim3 grid(T, (N + threads - 1) / threads);
+  DISTIE_DISPATCH(x_dtype, X, DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(out_dtype, O,
+      causal_conv_kernel<X, W, O><<<grid, threads, 0, stream>>>(
+          static_cast<const X*>(x), ldx, static_cast<const W*>(weight), taps, state, static_cast<O*>(out), ldo, residual,
+          cu_q, token_request, state_slots, N))));
+  return launch_status();
+}
+
+extern "C" int distie_conv_state(const void* x, int x_dtype, int64_t ldx, int taps, float* state, const int32_t* cu_q,
+                                 const int32_t* state_slots, int B, int N, int skip_single, hipStream_t stream) {
+  if (B <= 0 || taps <= 1) return 0;
+  if (taps > MAX_TAPS || N < 1 || ldx < N || state == nullptr) return DISTIE_BAD_ARGUMENT;
+  const int threads = N >= 256 ? 256 : (N >= 128 ? 128 : 64);
+  const dim3 grid(B, (N + threads - 1) / threads);
+  DISTIE_DISPATCH(x_dtype, X, conv_state_kernel<X><<<grid, threads, 0, stream>>>(
+      static_cast<const X*>(x), ldx, taps, state, cu_q, state_slots, N, skip_single));
+  return launch_status();
+}
+
+extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t ld, const void* weight, int w_dtype,
+                                         int taps, const float* state, const void* table, int pairs, float magnitude,
+                                         void* q_out, void* k_cache, void* v_cache, int cache_dtype, const int32_t* slots,
+                                         const int32_t* cu_q, const int32_t* token_request, const int32_t* state_slots,
+                                         int T, int H, int G, int D, int E, int DP, int block_size, int has_kv, int write,
+                                         hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H < 1 || G < 1 || D < 1 || E < 1 || DP < D || DP < E || block_size < 1 || pairs < 0 || 2 * pairs > D ||
+      taps < 0 || taps > MAX_TAPS)
+    return DISTIE_BAD_ARGUMENT;
+  if ((pairs > 0 && table == nullptr) || (taps > 1 && state == nullptr) || (taps >= 1 && weight == nullptr))
+    return DISTIE_BAD_ARGUMENT;
+  if (has_kv && write && (k_cache == nullptr || v_cache == nullptr || slots == nullptr)) return DISTIE_BAD_ARGUMENT;
+  const int work = (H + G) * DP;
+  const int threads = work >= 1024 ? 256 : (work >= 256 ? 128 : 64);
+  if (weight == nullptr) w_dtype = dtype;
+  DISTIE_DISPATCH(dtype, X, DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(cache_dtype, C,
+      conv_rope_kv_write_kernel<X, W, X, C><<<T, threads, 0, stream>>>(
+          static_cast<const X*>(product), ld, static_cast<const W*>(weight), taps, state, static_cast<const float2*>(table),
+          pairs, magnitude, static_cast<X*>(q_out), static_cast<C*>(k_cache), static_cast<C*>(v_cache), slots, cu_q,
+          token_request, state_slots, H, G, D, E, DP, block_size, has_kv, write))));
+  return launch_status();
+}
+
+extern "C" int distie_sigmoid_gate(const void* x, int x_dtype, int ldh, int E, const void* gates, int g_dtype, int64_t ldg,
+                                   void* out, int out_dtype, int T, int width, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (E < 1 || width < 1 || width % E || ldh < E || ldg < width) return DISTIE_BAD_ARGUMENT;
+  const int threads = width >= 256 ? 256 : (width >= 128 ? 128 : 64);
+  const dim3 grid(T, (width + threads - 1) / threads);
+  DISTIE_DISPATCH(x_dtype, X, DISTIE_DISPATCH(g_dtype, G, DISTIE_DISPATCH(out_dtype, O,
+      sigmoid_gate_kernel<X, G, O><<<grid, threads, 0, stream>>>(
+          static_cast<const X*>(x), ldh, E, static_cast<const G*>(gates), ldg, static_cast<O*>(out), width))));
+  return launch_status();
+}
+
+extern "C" int distie_rmsnorm_gate(const float* x, const void* weight, int w_dtype, float eps, const void* gates,
+                                   int g_dtype, int64_t ldg, void* out, int out_dtype, int T, int N, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (N < 1 || (gates != nullptr && ldg < N)) return DISTIE_BAD_ARGUMENT;
+  const int threads = N >= 2048 ? 512 : (N >= 512 ? 256 : (N >= 128 ? 128 : 64));
+  if (gates == nullptr) g_dtype = DISTIE_F32;
+  DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(g_dtype, G, DISTIE_DISPATCH(out_dtype, O,
+      rmsnorm_gate_kernel<W, G, O><<<T, threads, 0, stream>>>(
+          x, static_cast<const W*>(weight), eps, static_cast<const G*>(gates), ldg, static_cast<O*>(out), N))));
+  return launch_status();
+}
+
+extern "C" int distie_activation(const void* in, void* out, int dtype, int64_t count, int kind, hipStream_t stream) {
+  if (count <= 0) return 0;
+  if (kind < 0 || kind > 3) return DISTIE_BAD_ARGUMENT;
+  const int threads = 256;
+  const int64_t blocks = (count + threads - 1) / threads;
+  if (blocks > 0x7fffffff) return DISTIE_BAD_ARGUMENT;
+  DISTIE_DISPATCH(dtype, T, activation_kernel<T><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(
+      static_cast<const T*>(in), 1, 0, static_cast<T*>(out), count, kind));
+  return launch_status();
+}
+
+// the largest per-head key size the scan takes (rows of the state a thread keeps: PARTS x ROWS)
+extern "C" int distie_decay_scan_max_dim() { return 256; }
+
+extern "C" int distie_decay_scan(const void* product, int dtype, int64_t ld, float* state, const float* decay, float* out,
+                                 const int32_t* cu_q, const int32_t* state_slots, int B, int H, int D, int E,
+                                 hipStream_t stream) {
+  if (B <= 0) return 0;
+  if (H < 1 || D < 1 || E < 1 || D > 256 || ld < static_cast<int64_t>(H) * (2 * D + E)) return DISTIE_BAD_ARGUMENT;
+  const dim3 grid(B, H, (E + 63) / 64);
+#define DISTIE_SCAN(PARTS, ROWS)                                                                                     \
+  DISTIE_DISPATCH(dtype, X, decay_scan_kernel<X, PARTS, ROWS><<<grid, 64 * PARTS, 0, stream>>>(                      \
+      static_cast<const X*>(product), ld, state, decay, out, cu_q, state_slots, H, D, E))
+  if (D <= 32) {
+    DISTIE_SCAN(4, 8);
+  } else if (D <= 64) {
+    DISTIE_SCAN(4, 16);
+  } else if (D <= 128) {
+    DISTIE_SCAN(4, 32);
+  } else {
+    DISTIE_SCAN(8, 32);
+  }
+#undef DISTIE_SCAN
+  return launch_status();
+}

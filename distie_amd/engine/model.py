@@ -135,6 +135,7 @@ class Model:
             self.blocks[call.layer].forward(ops, stream, ctx, cache.layer(call.cache_layer), call.writes_cache)
         if want_rows is None:
             return None
+        stream.close(ops)            # an arrangement with a residual of its own form hands back the plain sum
         if every_row:
             normed = self.final_norm.of_stream(ops, stream, act_dtype)
             return self.lm_head.forward(ops, normed)

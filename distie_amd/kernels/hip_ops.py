@@ -292,6 +292,15 @@ class HipOps(Ops):
         o.distie_decode_product_residual.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
         o.distie_decode_norm_product.argtypes = [_P, _P, _F, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P,
                                                  _I, _I, _I, _I, _I, _P]
+        o.distie_hyper_step.argtypes = [_P, _I, _P, _P, _I, _I, _P, _I, _L, _P, _P, _P, _P, _I, _I, _F, _P, _I, _I, _I, _P]
+        o.distie_causal_conv.argtypes = [_P, _I, _L, _P, _I, _I, _P, _P, _I, _L, _I, _P, _P, _P, _I, _I, _P]
+        o.distie_conv_state.argtypes = [_P, _I, _L, _I, _P, _P, _P, _I, _I, _I, _P]
+        o.distie_conv_rope_kv_write.argtypes = [_P, _I, _L, _P, _I, _I, _P, _P, _I, _F, _P, _P, _P, _I, _P, _P, _P, _P,
+                                                _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]
+        o.distie_sigmoid_gate.argtypes = [_P, _I, _I, _I, _P, _I, _L, _P, _I, _I, _I, _P]
+        o.distie_rmsnorm_gate.argtypes = [_P, _P, _I, _F, _P, _I, _L, _P, _I, _I, _I, _P]
+        o.distie_activation.argtypes = [_P, _P, _I, _L, _I, _P]
+        o.distie_decay_scan.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]
         o.distie_argmax.argtypes = [_P, _P, _I, _I, _P, _P, _P]
         o.distie_argmax_parts.argtypes = [_I, _I]
         o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P]
@@ -996,6 +1005,182 @@ class HipOps(Ops):
             plan["prefill_o"] = torch.empty((parts, T, num_heads, head_dim), dtype=torch.float32, device=self.device)
             plan["prefill_ml"] = torch.empty((parts, T, num_heads, 2), dtype=torch.float32, device=self.device)
         return plan
+
+    # ---- residual streams, convolutions over time, decayed states, gates (csrc/sequence.hip)
+    def _rows_view(self, t: torch.Tensor, width: int):
+        """(pointer, row stride) of a [T, width] tensor or column view whose rows are contiguous."""
+        if t.device != self.device or t.dim() != 2 or t.shape[1] != width or (t.shape[1] > 1 and t.stride(1) != 1):
+            raise KernelError("kernels take row views with contiguous columns on their own device")
+        return t.data_ptr(), t.stride(0)
+
+    NORM_KINDS = {"none": 0, "layer": 1, "rms": 2}
+    ACTIVATIONS = {"relu2": 0, "silu": 1, "gelu_tanh": 2, "relu": 3}
+
+    def hyper_step(self, streams, *, init=None, delta=None, gate=None, mix=None, write=None, read=None,
+                   norm_weight=None, norm="none", eps=0.0, out_dtype=None):
+        if norm not in self.NORM_KINDS:
+            raise KernelError(f"no norm named {norm!r}")
+        if init is not None:
+            if streams is not None or mix is None and write is None and read is None:
+                raise KernelError("hyper_step: `init` makes the streams; it needs their number from mix, write or read")
+            self._own(init)
+            count = (read if read is not None else write).shape[0]
+            if init.dtype != torch.float32 or init.dim() != 2:
+                raise KernelError("hyper_step: init must be float32 [T, C]")
+            streams = torch.empty((init.shape[0], count, init.shape[1]), dtype=torch.float32, device=self.device)
+        self._own(streams, mix, write, read, norm_weight)
+        if streams.dtype != torch.float32 or streams.dim() != 3:
+            raise KernelError("hyper_step: streams must be float32 [T, S, C]")
+        T, S, C = streams.shape
+        for name, t, shape in (("mix", mix, (S, S)), ("write", write, (S,)), ("read", read, (S,))):
+            if t is not None and (t.dtype != torch.float32 or tuple(t.shape) != shape):
+                raise KernelError(f"hyper_step: {name} must be float32 {list(shape)}")
+        if init is not None and tuple(init.shape) != (T, C):
+            raise KernelError("hyper_step: init does not match the streams")
+        slices, y, y_code, g_ptr, g_code, g_ld = 1, None, _F32, None, _F32, 0
+        if delta is not None:
+            if mix is None or write is None:
+                raise KernelError("hyper_step: a delta needs mix and write weights")
+            if isinstance(delta, (PendingNorm, PendingProduct)):
+                delta = self.dense(delta)
+            if isinstance(delta, PartialSums):
+                slices, delta = delta.slices, delta.data
+            self._own(delta)
+            if tuple(delta.shape[-2:]) != (T, C):
+                raise KernelError("hyper_step: delta must be [T, C]")
+            y, y_code = delta.data_ptr(), _code(delta)
+            if gate is not None:
+                g_ptr, g_ld = self._rows_view(gate, C)
+                g_code = _code(gate)
+        h = None
+        if read is not None:
+            if norm != "none" and (norm_weight is None or tuple(norm_weight.shape) != (C,)):
+                raise KernelError("hyper_step: the norm needs a weight [C]")
+            h = torch.empty((T, C), dtype=out_dtype or torch.float32, device=self.device)
+        ptr = lambda t: t.data_ptr() if t is not None else None
+        _check(self._ops.distie_hyper_step(
+            streams.data_ptr(), S, ptr(init), y, y_code, slices, g_ptr, g_code, g_ld, ptr(mix), ptr(write), ptr(read),
+            ptr(norm_weight), _code(norm_weight) if norm_weight is not None else _F32, self.NORM_KINDS[norm], float(eps),
+            ptr(h), _code(h) if h is not None else _F32, T, C, self._stream()), "hyper_step")
+        _mark_written(streams)
+        return streams, h
+
+    def causal_conv(self, x, weight, state, meta, residual=False):
+        x = self.dense(x)
+        self._own(x, weight, state)
+        T, N = x.shape
+        taps = weight.shape[1]
+        if tuple(weight.shape) != (N, taps) or T != meta.num_tokens:
+            raise KernelError("causal_conv: weight must be [channels of x, taps], x the step's rows")
+        self._check_conv_state(state, taps, N)
+        out = torch.empty_like(x)
+        _check(self._ops.distie_causal_conv(
+            x.data_ptr(), _code(x), N, weight.data_ptr(), _code(weight), taps, state.data_ptr() if taps > 1 else None,
+            out.data_ptr(), _code(out), N, 1 if residual else 0, meta.cu_q.data_ptr(), meta.token_request.data_ptr(),
+            meta.state_slots.data_ptr(), T, N, self._stream()), "causal_conv")
+        if taps > 1 and not meta.all_decode:
+            # requests that bring one row moved their state on in the kernel above; the others here, once all
+            # rows of the step have read the old one
+            _check(self._ops.distie_conv_state(x.data_ptr(), _code(x), N, taps, state.data_ptr(), meta.cu_q.data_ptr(),
+                                               meta.state_slots.data_ptr(), meta.num_requests, N, 1, self._stream()),
+                   "conv_state")
+        if taps > 1:
+            _mark_written(state)
+        return out
+
+    def _check_conv_state(self, state, taps, channels) -> None:
+        if taps > 1 and (state is None or state.dtype != torch.float32 or tuple(state.shape[1:]) != (taps - 1, channels)):
+            raise KernelError(f"the state of a convolution of {taps} taps over {channels} channels is float32 "
+                              f"[slots, {taps - 1}, {channels}]")
+
+    def conv_rope_kv_write(self, product, conv_weight, state, meta, group, k_cache, v_cache, inv_freq, magnitude,
+                           num_heads, num_kv_heads, dim, value_dim, padded_dim, has_kv, write):
+        product = self.dense(product)
+        self._own(product, conv_weight, state, k_cache, v_cache, inv_freq)
+        T, W = product.shape
+        channels = num_heads * dim + (num_kv_heads * (dim + value_dim) if has_kv else 0)
+        taps = 0 if conv_weight is None else conv_weight.shape[1]
+        if T != meta.num_tokens or W < channels:
+            raise KernelError("conv_rope_kv_write: the product does not match the batch or the head counts")
+        if conv_weight is not None and tuple(conv_weight.shape) != (channels, taps):
+            raise KernelError(f"conv_rope_kv_write: the filters must be [{channels}, taps]")
+        self._check_conv_state(state, taps, channels)
+        write = bool(write and has_kv)
+        if write:
+            self._check_cache(k_cache, v_cache, num_kv_heads, meta.block_size, padded_dim)
+            if k_cache.dtype != v_cache.dtype:
+                raise KernelError("conv_rope_kv_write: keys and values are cached in one dtype")
+        pairs = 0 if inv_freq is None else inv_freq.shape[0]
+        table = self._rope_table(meta, inv_freq) if pairs else None
+        q = torch.empty((T, num_heads * padded_dim), dtype=product.dtype, device=self.device)
+        ptr = lambda t: t.data_ptr() if t is not None else None
+        _check(self._ops.distie_conv_rope_kv_write(
+            product.data_ptr(), _code(product), W, ptr(conv_weight), _code(conv_weight) if conv_weight is not None else _F32,
+            taps, ptr(state) if taps > 1 else None, ptr(table), pairs, float(magnitude), q.data_ptr(),
+            ptr(k_cache) if write else None, ptr(v_cache) if write else None, _code(k_cache) if write else _code(product),
+            meta.groups[group].slots.data_ptr() if write else None, meta.cu_q.data_ptr(), meta.token_request.data_ptr(),
+            meta.state_slots.data_ptr(), T, num_heads, num_kv_heads, dim, value_dim, padded_dim, meta.block_size,
+            1 if has_kv else 0, 1 if write else 0, self._stream()), "conv_rope_kv_write")
+        if taps > 1:
+            _check(self._ops.distie_conv_state(product.data_ptr(), _code(product), W, taps, state.data_ptr(),
+                                               meta.cu_q.data_ptr(), meta.state_slots.data_ptr(), meta.num_requests,
+                                               channels, 0, self._stream()), "conv_state")
+            _mark_written(state)
+        return q
+
+    def sigmoid_gate(self, x, num_heads, head_stride, width, gates):
+        x = self.dense(x)
+        self._own(x)
+        T = x.shape[0]
+        if x.shape[1] != num_heads * head_stride or width > head_stride:
+            raise KernelError("sigmoid_gate: x must be [T, heads * head_stride]")
+        g_ptr, g_ld = self._rows_view(gates, num_heads * width)
+        out = torch.empty((T, num_heads * width), dtype=x.dtype, device=self.device)
+        _check(self._ops.distie_sigmoid_gate(x.data_ptr(), _code(x), head_stride, width, g_ptr, _code(gates), g_ld,
+                                             out.data_ptr(), _code(out), T, num_heads * width, self._stream()),
+               "sigmoid_gate")
+        return out
+
+    def decay_scan(self, product, state, decay, meta, num_heads, dim, value_dim):
+        product = self.dense(product)
+        self._own(product, state, decay)
+        T, W = product.shape
+        if T != meta.num_tokens or W < num_heads * (2 * dim + value_dim):
+            raise KernelError("decay_scan: the product does not match the batch or the head counts")
+        if state.dtype != torch.float32 or tuple(state.shape[1:]) != (num_heads, dim, value_dim):
+            raise KernelError("decay_scan: the state is float32 [slots, heads, dim, value_dim]")
+        if decay.dtype != torch.float32 or tuple(decay.shape) != (num_heads,):
+            raise KernelError("decay_scan: decay must be float32 [heads]")
+        out = torch.empty((T, num_heads * value_dim), dtype=torch.float32, device=self.device)
+        _check(self._ops.distie_decay_scan(product.data_ptr(), _code(product), W, state.data_ptr(), decay.data_ptr(),
+                                           out.data_ptr(), meta.cu_q.data_ptr(), meta.state_slots.data_ptr(),
+                                           meta.num_requests, num_heads, dim, value_dim, self._stream()), "decay_scan")
+        _mark_written(state)
+        return out
+
+    def rmsnorm_gate(self, x, weight, eps, gates, out_dtype):
+        self._own(x, weight)
+        if x.dtype != torch.float32 or x.dim() != 2 or tuple(weight.shape) != (x.shape[1],):
+            raise KernelError("rmsnorm_gate: x must be float32 [T, N], weight [N]")
+        T, N = x.shape
+        g_ptr, g_ld, g_code = None, 0, _F32
+        if gates is not None:
+            g_ptr, g_ld = self._rows_view(gates, N)
+            g_code = _code(gates)
+        out = torch.empty((T, N), dtype=out_dtype, device=self.device)
+        _check(self._ops.distie_rmsnorm_gate(x.data_ptr(), weight.data_ptr(), _code(weight), float(eps), g_ptr, g_code,
+                                             g_ld, out.data_ptr(), _code(out), T, N, self._stream()), "rmsnorm_gate")
+        return out
+
+    def activation(self, x, kind):
+        if kind not in self.ACTIVATIONS:
+            raise KernelError(f"no activation named {kind!r}")
+        x = self.dense(x)
+        self._own(x)
+        out = torch.empty_like(x)
+        _check(self._ops.distie_activation(x.data_ptr(), out.data_ptr(), _code(x), x.numel(), self.ACTIVATIONS[kind],
+                                           self._stream()), "activation")
+        return out
 
     def silu_mul(self, gate_up):
         if isinstance(gate_up, (PendingNorm, PendingProduct)):

@@ -179,6 +179,81 @@ class Ops(abc.ABC):
         `window` of them on a windowed layer), read through the block table -> act [T, H*D].
         `extras`: what a variant adds to the scores (`ScoreExtras`); None for plain attention."""
 
+    # ---- several residual streams, short convolutions over time, decayed states, gates. An implementation that
+    # ---- serves only models without them may leave these out: the bodies here refuse.
+    def hyper_step(self, streams: Optional[torch.Tensor], *, init: Optional[torch.Tensor] = None, delta=None,
+                   gate: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None,
+                   write: Optional[torch.Tensor] = None, read: Optional[torch.Tensor] = None,
+                   norm_weight: Optional[torch.Tensor] = None, norm: str = "none", eps: float = 0.0, out_dtype=None):
+        """One step on S residual streams, float32 [T, S, C], updated in place -> (streams, h or None).
+
+        `init` (float32 [T, C]): the streams do not exist yet and all start as `init` (`streams` is None).
+        `delta` (act [T, C], with `mix` float32 [S, S] indexed [from, to] and `write` float32 [S]): all streams
+        at once from the old ones, x_j <- sum_s mix[s, j] x_s + write[j] * delta * sigmoid(gate) (`gate` act
+        [T, C] or a view with a row stride; None: no gate). `read` (float32 [S]): h = norm(sum_s read[s] x_s)
+        * norm_weight in `out_dtype`, from the updated streams; `norm` is "none" (h is the sum, float32 unless
+        `out_dtype` says otherwise), "layer" ((u - mean) / sqrt(var + eps), var the mean of the squared deviations)
+        or "rms" (u / sqrt(mean(u^2) + eps)). Statistics and sums in float32."""
+        raise NotImplementedError(f"{type(self).__name__} has no residual streams")
+
+    def layernorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+        """float32 [T, C] -> (x - mean) / sqrt(var + eps) * weight, no bias, statistics in float32."""
+        ones = torch.ones(1, dtype=torch.float32, device=x.device)
+        return self.hyper_step(x.view(x.shape[0], 1, x.shape[1]), read=ones, norm_weight=weight, norm="layer",
+                               eps=eps, out_dtype=out_dtype)[1]
+
+    def causal_conv(self, x: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor], meta: BatchMeta,
+                    residual: bool = False) -> torch.Tensor:
+        """x act [T, N], weight [N, taps] -> y_t = (x_t if residual) + sum_j weight[:, j] * x_(t - taps + 1 + j)
+        within each request; what lies before the step's rows comes from `state` (float32 [slots + 1, taps - 1, N],
+        the request's last taps - 1 inputs, oldest first, rows by `meta.state_slots`), which is moved on to the
+        end of the step's rows. Sums in float32, in the order of j."""
+        raise NotImplementedError(f"{type(self).__name__} has no convolution over time")
+
+    def conv_rope_kv_write(self, product: torch.Tensor, conv_weight: Optional[torch.Tensor],
+                           state: Optional[torch.Tensor], meta: BatchMeta, group: int,
+                           k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                           inv_freq: Optional[torch.Tensor], magnitude: float, num_heads: int, num_kv_heads: int,
+                           dim: int, value_dim: int, padded_dim: int, has_kv: bool, write: bool) -> torch.Tensor:
+        """Behind attention's stacked projection. The first columns of `product` (act [T, W]) are q (num_heads x
+        dim) and, if `has_kv`, k (num_kv_heads x dim) and v (num_kv_heads x value_dim); further columns are left
+        alone. Each of these channels goes through `causal_conv` (no residual; `conv_weight` [channels, taps],
+        None: no convolution; the state is moved on), the first 2 * len(inv_freq) dimensions of every q and k head
+        are rotated by the token's position (pair (i, i + len(inv_freq)); cosine and sine both times
+        `magnitude`), and, if `write`, k and v go to the token's slot of k_cache [pages, KH, P, padded_dim] /
+        v_cache [pages, KH, padded_dim, P]. Returns q as act [T, num_heads * padded_dim], zeros beyond `dim`:
+        what `paged_attention` reads with a head size of `padded_dim`."""
+        raise NotImplementedError(f"{type(self).__name__} has no convolution over time")
+
+    def sigmoid_gate(self, x: torch.Tensor, num_heads: int, head_stride: int, width: int,
+                     gates: torch.Tensor) -> torch.Tensor:
+        """x act [T, num_heads * head_stride], of which the first `width` of every head count; gates act
+        [T, num_heads * width] (or a view with a row stride) -> x * sigmoid(gates), act [T, num_heads * width]."""
+        raise NotImplementedError(f"{type(self).__name__} has no gates")
+
+    def decay_scan(self, product: torch.Tensor, state: torch.Tensor, decay: torch.Tensor, meta: BatchMeta,
+                   num_heads: int, dim: int, value_dim: int) -> torch.Tensor:
+        """Linear attention with a decay per head, as a recurrence over each request's rows: with q = silu(.),
+        k = silu(.) (num_heads x dim each) and v = silu(.) (num_heads x value_dim) taken from the first columns of
+        `product` (act [T, W]), S <- decay[h] * S + k v^T and o = S^T q. `state` float32 [slots + 1, num_heads,
+        dim, value_dim] (rows by `meta.state_slots`) is read and left as the step's last row leaves it.
+        -> float32 [T, num_heads * value_dim]. Everything behind the activations in float32."""
+        raise NotImplementedError(f"{type(self).__name__} has no decayed state")
+
+    def rmsnorm_gate(self, x: torch.Tensor, weight: torch.Tensor, eps: float, gates: Optional[torch.Tensor],
+                     out_dtype) -> torch.Tensor:
+        """float32 [T, N] -> x / sqrt(mean(x^2) + eps) * weight * sigmoid(gates) in `out_dtype` (gates act [T, N]
+        or a view with a row stride; None: no gate)."""
+        raise NotImplementedError(f"{type(self).__name__} has no gated norm")
+
+    def activation(self, x, kind: str) -> torch.Tensor:
+        """Element by element on act [T, N]: "relu2" (the square of max(x, 0)), "silu", "gelu_tanh", "relu"."""
+        raise NotImplementedError(f"{type(self).__name__} has no activation {kind!r}")
+
+    def linear_act(self, x, weight: torch.Tensor, kind: str) -> torch.Tensor:
+        """activation(linear(x, weight), kind); an implementation may fuse the two."""
+        return self.activation(self.linear(x, weight), kind)
+
     @abc.abstractmethod
     def silu_mul(self, gate_up: torch.Tensor) -> torch.Tensor:
         """[T, 2I] -> silu(first half) * second half, [T, I]."""

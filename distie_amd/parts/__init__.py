@@ -1,8 +1,9 @@
-from . import attention, block, embedding, feed_forward, norm, position  # noqa: F401  (registration)
+from . import (attention, block, conv_attention, embedding, feed_forward, linear_attention, norm,  # noqa: F401  (registration)
+               position)
 from .attention import PagedKV
-from .base import (PAGE, Block, Embedding, FeedForward, FixedState, Head, Mixer, Norm, PagedTensors, ParamSpec, Part,
+from .base import (PAGE, Block, Borrowed, CacheNeeds, Embedding, FeedForward, FixedState, Head, Mixer, Norm, PagedTensors, ParamSpec, Part,
                    PositionEncoding, ResidualStream, StepContext, TensorDecl, build_part, register_part)
 
-__all__ = ["PAGE", "Block", "Embedding", "FeedForward", "FixedState", "Head", "Mixer", "Norm", "PagedKV", "PagedTensors",
+__all__ = ["PAGE", "Block", "Borrowed", "CacheNeeds", "Embedding", "FeedForward", "FixedState", "Head", "Mixer", "Norm", "PagedKV", "PagedTensors",
            "ParamSpec", "Part", "PositionEncoding", "ResidualStream", "StepContext", "TensorDecl", "build_part",
            "register_part"]

@@ -83,6 +83,24 @@ class FixedState:
         return cls((TensorDecl(name, tuple(shape), torch.float32),))
 
 
+@dataclass(frozen=True)
+class Borrowed:
+    """A mixer that keeps no pages of its own: it reads those of mixer `name` of layer `layer` (which must keep
+    them for as long as this mixer looks back) and writes nothing there."""
+
+    layer: int
+    name: str = "mixer"
+
+
+@dataclass(frozen=True)
+class CacheNeeds:
+    """What a part keeps when it is more than one thing: pages (its own, or another mixer's) and tensors of fixed
+    size per request. The part's view holds all of them by name."""
+
+    paged: Optional[object] = None          # PagedTensors | Borrowed
+    state: Optional[FixedState] = None
+
+
 class ResidualStream:
     """The residual sum in float32, and a contribution not yet added to it. The next norm
     adds it while it reads the stream, which saves one pass over the activations."""
@@ -90,6 +108,16 @@ class ResidualStream:
     def __init__(self, hidden: torch.Tensor) -> None:
         self.hidden = hidden
         self.pending: Optional[torch.Tensor] = None
+        # An arrangement that keeps the residual in a form of its own (several streams) hangs it here, with a
+        # function that turns it back into `hidden` [T, C] and `pending` once the last block has run.
+        self.lanes = None
+        self.settle: Optional[Callable] = None
+
+    def close(self, ops) -> None:
+        """After the last block: `hidden` (and `pending`) are the plain residual sum again."""
+        if self.settle is not None:
+            settle, self.settle = self.settle, None
+            settle(ops, self)
 
 
 class StepContext:
@@ -173,6 +201,10 @@ class PositionEncoding(Part):
         cache write, or None if this encoding does not rotate."""
         return None
 
+    def rotary_magnitude(self) -> float:
+        """What cosine and sine of the rotation are both multiplied by (1 for a plain rotation)."""
+        return 1.0
+
     def head_slopes(self, num_heads: int) -> Optional[torch.Tensor]:
         """float32 [num_heads] for an encoding that biases every score by the distance to the key,
         score += slope[h] * (key position - query position) (`ScoreExtras.head_slopes`); None otherwise."""
@@ -204,16 +236,20 @@ class Block(Part):
     built here and becomes an attribute of its name."""
 
     CHILDREN: Dict[str, str] = {}
+    OPTIONAL: Tuple[str, ...] = ()          # children a layer may leave out (the attribute is then None)
 
     def __init__(self, spec: PartSpec, parts: Mapping[str, PartSpec]) -> None:
         super().__init__(spec)
-        missing = [name for name in self.CHILDREN if name not in parts]
+        missing = [name for name in self.CHILDREN if name not in parts and name not in self.OPTIONAL]
         unknown = [name for name in parts if name not in self.CHILDREN]
         if missing or unknown:
             raise ValueError(f"block {spec.kind!r} arranges {sorted(self.CHILDREN)}: "
                              f"missing {missing}, not known to it {unknown}")
         self.children: Dict[str, Part] = {}
         for name, family in self.CHILDREN.items():
+            if name not in parts:
+                setattr(self, name, None)
+                continue
             child = build_part(family, parts[name])
             self.children[name] = child
             setattr(self, name, child)
@@ -224,7 +260,9 @@ class Block(Part):
         yield self
 
     def cache_requirements(self) -> Dict[str, object]:
-        """What each of the block's mixers keeps, by the mixer's name in the block."""
+        """What each of the block's mixers keeps, by the mixer's name in the block. An arrangement that keeps
+        something itself (the last inputs of a convolution in front of a sub-layer) adds it under a name of
+        its own; `forward` finds it as `cache[name]`."""
         return {name: child.cache_requirement() for name, child in self.children.items()
                 if self.CHILDREN[name] == "mixer"}
 

@@ -13,13 +13,14 @@ class TokenEmbedding(Embedding):
         super().__init__(spec)
         self.vocab_size = int(spec.params["vocab_size"])
         self.hidden_size = int(spec.params["hidden_size"])
+        self.weight_name = spec.params.get("weight_name", "weight")      # the tensor's name behind the prefix
         self.weight = None
 
     def param_specs(self):
-        return {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+        return {self.weight_name: ParamSpec((self.vocab_size, self.hidden_size))}
 
     def load(self, tensors) -> None:
-        self.weight = tensors["weight"].contiguous()
+        self.weight = tensors[self.weight_name].contiguous()
 
     def forward(self, ops, ids, meta):
         return ops.embed(ids, self.weight)
@@ -31,19 +32,20 @@ class LinearHead(Head):
         self.vocab_size = int(spec.params["vocab_size"])
         self.hidden_size = int(spec.params["hidden_size"])
         self.tied_to = spec.params.get("tied_to")        # full name of the tensor to share, or None
+        self.weight_name = spec.params.get("weight_name", "weight")
         self.weight = None
 
     def param_specs(self):
-        return {} if self.tied_to else {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+        return {} if self.tied_to else {self.weight_name: ParamSpec((self.vocab_size, self.hidden_size))}
 
     def shared_specs(self):
-        return {"weight": self.tied_to} if self.tied_to else {}
+        return {self.weight_name: self.tied_to} if self.tied_to else {}
 
     def optional_names(self):
-        return ["weight"] if self.tied_to else []
+        return [self.weight_name] if self.tied_to else []
 
     def load(self, tensors) -> None:
-        self.weight = tensors["weight"] if self.tied_to else tensors["weight"].contiguous()
+        self.weight = tensors[self.weight_name] if self.tied_to else tensors[self.weight_name].contiguous()
 
     def prepare(self, ops) -> None:
         ops.prepare_linear(self.weight, role="head")

@@ -1,13 +1,17 @@
-"""RMS norm: y = weight * x * rsqrt(mean(x^2) + eps), statistics in float32
+"""Norms. RMS norm: y = weight * x * rsqrt(mean(x^2) + eps), statistics in float32
 (worker/src/inference/qwen2/model.py:77-90). The reference multiplies by the weight
 after rounding back to the model dtype; here the product is rounded once."""
 
 from __future__ import annotations
 
+import torch
+
 from .base import Norm, ParamSpec, register_part
 
 
 class RMSNorm(Norm):
+    fused_kind = "rms"          # what `Ops.hyper_step` calls this norm when it computes it while reading the streams
+
     def __init__(self, spec) -> None:
         super().__init__(spec)
         self.size = int(spec.params["size"])
@@ -27,4 +31,34 @@ class RMSNorm(Norm):
         return ops.add_rmsnorm(residual, delta, self.weight, self.eps, out_dtype)
 
 
+class LayerNorm(Norm):
+    """Centred norm with a weight and no bias: y = (x - mean) / sqrt(var + eps) * weight, where var is the mean of
+    the squared deviations; statistics in float32."""
+
+    fused_kind = "layer"
+
+    def __init__(self, spec) -> None:
+        super().__init__(spec)
+        self.size = int(spec.params["size"])
+        self.eps = float(spec.params["eps"])
+        self.weight = None
+        self._one = None
+
+    def param_specs(self):
+        return {self.spec.params.get("weight_name", "weight"): ParamSpec((self.size,), "ones")}
+
+    def load(self, tensors) -> None:
+        self.weight = tensors[self.spec.params.get("weight_name", "weight")].contiguous()
+        self._one = torch.ones(1, dtype=torch.float32, device=self.weight.device)
+
+    def apply(self, ops, x, out_dtype):
+        return ops.layernorm(x, self.weight, self.eps, out_dtype)
+
+    def add_apply(self, ops, residual, delta, out_dtype):
+        rows, width = residual.shape
+        return ops.hyper_step(residual.view(rows, 1, width), delta=delta, mix=self._one.view(1, 1), write=self._one,
+                              read=self._one, norm_weight=self.weight, norm="layer", eps=self.eps, out_dtype=out_dtype)[1]
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "layernorm", LayerNorm)

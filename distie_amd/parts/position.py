@@ -5,6 +5,8 @@ float32 inside the kernel that also writes the cache."""
 
 from __future__ import annotations
 
+import math
+
 import torch
 
 from .base import PositionEncoding, register_part
@@ -36,9 +38,59 @@ class RotaryPosition(PositionEncoding):
         return self.inv_freq
 
 
+class ScaledRotaryPosition(PositionEncoding):
+    """Rotation of the first `dims` dimensions of a head, with the frequencies stretched for contexts beyond the
+    trained one ("YaRN"): f_i = base^(-2i/dims); with `scaling` = {factor, original, fast, slow}, the dimension at
+    which a frequency makes `turns` turns over `original` positions is dim(turns) = dims ln(original / (2 pi turns))
+    / (2 ln base); lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), dims - 1), ramp_i = clamp((i - lo) /
+    max(hi - lo, 0.001), 0, 1), and the frequency becomes f_i / factor * ramp_i + f_i * (1 - ramp_i): fast
+    dimensions keep theirs, slow ones are divided by the factor. Cosine and sine are both multiplied by
+    0.1 ln(factor) + 1 (`rotary_magnitude`). Without `scaling`: plain rotation of `dims` dimensions."""
+
+    def __init__(self, spec) -> None:
+        super().__init__(spec)
+        p = spec.params
+        self.dims = int(p["dims"])
+        self.base = float(p["base"])
+        if self.dims < 2 or self.dims % 2:
+            raise ValueError("rotary dimension must be even")
+        half = self.dims // 2
+        freq = torch.tensor([self.base ** (-2.0 * i / self.dims) for i in range(half)], dtype=torch.float64)
+        self.magnitude = 1.0
+        scaling = p.get("scaling")
+        if scaling:
+            factor, original = float(scaling["factor"]), float(scaling["original"])
+            fast, slow = float(scaling["fast"]), float(scaling["slow"])
+
+            def dim_of(turns: float) -> float:
+                return self.dims * math.log(original / (2 * math.pi * turns)) / (2 * math.log(self.base))
+
+            lo = max(math.floor(dim_of(fast)), 0)
+            hi = min(math.ceil(dim_of(slow)), self.dims - 1)
+            ramp = torch.tensor([min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0) for i in range(half)],
+                                dtype=torch.float64)
+            freq = freq / factor * ramp + freq * (1 - ramp)
+            self.magnitude = 0.1 * math.log(factor) + 1.0
+        self.inv_freq = freq.to(torch.float32)
+        self._key = (self.dims, self.base, repr(sorted(scaling.items())) if scaling else None)
+
+    def to_device(self, device) -> None:
+        key = ("scaled",) + self._key + (str(device),)
+        if key not in _SHARED:
+            _SHARED[key] = self.inv_freq.to(device)
+        self.inv_freq = _SHARED[key]
+
+    def rotary(self):
+        return self.inv_freq
+
+    def rotary_magnitude(self) -> float:
+        return self.magnitude
+
+
 class NoPosition(PositionEncoding):
     """For mixers whose order comes from elsewhere (a state, a learned table)."""
 
 
 register_part("position", "rope", RotaryPosition)
+register_part("position", "rope_scaled", ScaledRotaryPosition)
 register_part("position", "none", NoPosition)

@@ -63,7 +63,7 @@ class TorchOps(Ops):
                         scale, window, extras=None):
         T = qkv.shape[0]
         P = k_cache.shape[2]
-        q_all = qkv.view(T, num_heads + 2 * num_kv_heads, head_dim)[:, :num_heads].float()
+        q_all = qkv[:, :num_heads * head_dim].reshape(T, num_heads, head_dim).float()      # (q may come without k and v)
         out = torch.zeros(T, num_heads, head_dim, dtype=torch.float32, device=qkv.device)
         table = meta.groups[group].block_table.long()
         if meta.table_rows is not None:
@@ -88,6 +88,123 @@ class TorchOps(Ops):
                     s = s + extras.head_slopes.float()[:, None] * (keys - pos).float()[None, :]
                 out[t] = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), v)
         return out.view(T, num_heads * head_dim).to(qkv.dtype)
+
+    # ---- residual streams, convolutions over time, decayed states, gates
+    def hyper_step(self, streams, *, init=None, delta=None, gate=None, mix=None, write=None, read=None,
+                   norm_weight=None, norm="none", eps=0.0, out_dtype=None):
+        if init is not None:
+            count = (read if read is not None else write).shape[0]
+            streams = init.float()[:, None, :].repeat(1, count, 1)
+        if delta is not None:
+            d = delta.float()
+            if gate is not None:
+                d = d * torch.sigmoid(gate.float())
+            streams.copy_(torch.einsum("sj,tsc->tjc", mix.float(), streams) + write.float()[None, :, None] * d[:, None, :])
+        h = None
+        if read is not None:
+            u = torch.einsum("s,tsc->tc", read.float(), streams)
+            if norm == "layer":
+                mean = u.mean(-1, keepdim=True)
+                u = (u - mean) / torch.sqrt(((u - mean) ** 2).mean(-1, keepdim=True) + eps) * norm_weight.float()
+            elif norm == "rms":
+                u = u / torch.sqrt((u ** 2).mean(-1, keepdim=True) + eps) * norm_weight.float()
+            h = u.to(out_dtype or torch.float32)
+        return streams, h
+
+    def _history(self, x, state, meta, taps):
+        """Per request: (rows of the step, its state row, the inputs with the state in front)."""
+        cu = meta.cu_q.tolist()
+        slots = meta.state_slots.tolist()
+        for b in range(meta.num_requests):
+            rows = slice(cu[b], cu[b + 1])
+            past = state[slots[b]] if taps > 1 else x.new_zeros((0, x.shape[1]), dtype=torch.float32)
+            yield rows, slots[b], torch.cat([past, x[rows].float()], 0)
+
+    def _conv(self, x, weight, state, meta, residual):
+        taps = weight.shape[1]
+        out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+        for rows, slot, full in self._history(x, state, meta, taps):
+            n = rows.stop - rows.start
+            for j in range(taps):
+                out[rows] += weight[:, j].float() * full[j:j + n]
+            if taps > 1:
+                state[slot] = full[-(taps - 1):]
+        if residual:
+            out += x.float()
+        return out
+
+    def causal_conv(self, x, weight, state, meta, residual=False):
+        return self._conv(x, weight, state, meta, residual).to(x.dtype)
+
+    def conv_rope_kv_write(self, product, conv_weight, state, meta, group, k_cache, v_cache, inv_freq, magnitude,
+                           num_heads, num_kv_heads, dim, value_dim, padded_dim, has_kv, write):
+        T = product.shape[0]
+        channels = num_heads * dim + (num_kv_heads * (dim + value_dim) if has_kv else 0)
+        u = product[:, :channels]
+        u = self._conv(u, conv_weight, state, meta, False) if conv_weight is not None else u.float()
+        u = u.to(product.dtype).float()                   # the convolution's result in the activations' precision
+
+        def turned(x):
+            if inv_freq is None:
+                return x
+            pairs = inv_freq.shape[0]
+            ang = meta.positions.float()[:, None] * inv_freq.float()[None, :]
+            cos, sin = (ang.cos() * magnitude)[:, None, :], (ang.sin() * magnitude)[:, None, :]
+            a, b = x[..., :pairs], x[..., pairs:2 * pairs]
+            return torch.cat([a * cos - b * sin, b * cos + a * sin, x[..., 2 * pairs:]], -1)
+
+        q = torch.zeros(T, num_heads, padded_dim, dtype=torch.float32, device=product.device)
+        q[..., :dim] = turned(u[:, :num_heads * dim].view(T, num_heads, dim))
+        if has_kv and write:
+            k = turned(u[:, num_heads * dim:(num_heads + num_kv_heads) * dim].view(T, num_kv_heads, dim))
+            v = u[:, (num_heads + num_kv_heads) * dim:].view(T, num_kv_heads, value_dim)
+            P = k_cache.shape[2]
+            slots = meta.groups[group].slots.long()
+            k_cache[slots // P, :, slots % P, :dim] = k.to(k_cache.dtype)
+            v_cache[slots // P, :, :value_dim, slots % P] = v.to(v_cache.dtype)
+        return q.view(T, num_heads * padded_dim).to(product.dtype)
+
+    def sigmoid_gate(self, x, num_heads, head_stride, width, gates):
+        T = x.shape[0]
+        kept = x.view(T, num_heads, head_stride)[..., :width].reshape(T, num_heads * width).float()
+        return (kept * torch.sigmoid(gates.float())).to(x.dtype)
+
+    def decay_scan(self, product, state, decay, meta, num_heads, dim, value_dim):
+        T = product.shape[0]
+        act = lambda z: z * torch.sigmoid(z)
+        q = act(product[:, :num_heads * dim].float()).view(T, num_heads, dim)
+        k = act(product[:, num_heads * dim:2 * num_heads * dim].float()).view(T, num_heads, dim)
+        v = act(product[:, 2 * num_heads * dim:num_heads * (2 * dim + value_dim)].float()).view(T, num_heads, value_dim)
+        out = torch.zeros(T, num_heads, value_dim, dtype=torch.float32, device=product.device)
+        cu = meta.cu_q.tolist()
+        slots = meta.state_slots.tolist()
+        for b in range(meta.num_requests):
+            s = state[slots[b]]
+            for t in range(cu[b], cu[b + 1]):
+                s = decay.float()[:, None, None] * s + k[t][:, :, None] * v[t][:, None, :]
+                out[t] = torch.einsum("hde,hd->he", s, q[t])
+            state[slots[b]] = s
+        return out.view(T, num_heads * value_dim)
+
+    def rmsnorm_gate(self, x, weight, eps, gates, out_dtype):
+        y = x / torch.sqrt((x ** 2).mean(-1, keepdim=True) + eps) * weight.float()
+        if gates is not None:
+            y = y * torch.sigmoid(gates.float())
+        return y.to(out_dtype)
+
+    def activation(self, x, kind):
+        z = x.float()
+        if kind == "relu2":
+            r = torch.relu(z) ** 2
+        elif kind == "silu":
+            r = z * torch.sigmoid(z)
+        elif kind == "gelu_tanh":
+            r = 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
+        elif kind == "relu":
+            r = torch.relu(z)
+        else:
+            raise ValueError(kind)
+        return r.to(x.dtype)
 
     def silu_mul(self, gate_up):
         inter = gate_up.shape[1] // 2
