@@ -6,8 +6,8 @@ As in the reference (worker/src/inference/qwen2/batch_decode.py:42-211): batch s
 rounded up to a bucket (1, 2, 4, 8, then steps of 8, and the maximum); each bucket has its
 own fixed device buffers that the graph reads (tokens, positions, tables, slots) and its own
 logits; rows added to fill the bucket write to the sink page; a bucket is captured the first
-time it is used, after one ordinary run with the same buffers (so that scratch memory has
-its size and the first result is right), and replayed from then on. If capture or replay
+time it is used, behind one ordinary run with the same buffers (which is that step: a step runs
+once, since a mixer may carry a state that a second run would move on again), and replayed from then on. If capture or replay
 fails, the graphs and the memory pool they share are dropped, the step runs the ordinary way
 (which writes the same cache slots again), and so do the next decode steps; later a capture is
 tried again, and after a few failures captured steps stay off. Failures are counted and logged.
@@ -195,14 +195,17 @@ class DecodeGraphs:
         try:
             return self._run(bucket, entries, feed, max_kv)
         except Exception:  # noqa: BLE001 - the ordinary path rewrites the same slots
-            self.failures += 1
-            self._resting = self.RETRY_AFTER_STEPS
-            self.drop()
-            _log.exception("captured step failed (failure %d of %d allowed): graphs and their memory pool "
-                           "are dropped, steps run uncaptured %s", self.failures, self.MAX_FAILURES,
-                           "from now on" if self.failures >= self.MAX_FAILURES
-                           else f"for the next {self.RETRY_AFTER_STEPS} steps that a graph would take")
+            self._note_failure()
             return None
+
+    def _note_failure(self) -> None:
+        self.failures += 1
+        self._resting = self.RETRY_AFTER_STEPS
+        self.drop()
+        _log.exception("captured step failed (failure %d of %d allowed): graphs and their memory pool "
+                       "are dropped, steps run uncaptured %s", self.failures, self.MAX_FAILURES,
+                       "from now on" if self.failures >= self.MAX_FAILURES
+                       else f"for the next {self.RETRY_AFTER_STEPS} steps that a graph would take")
 
     def _run(self, bucket: _Bucket, entries: Sequence[StepEntry], feed: Optional[torch.Tensor],
              max_kv: int) -> Optional[torch.Tensor]:
@@ -263,12 +266,15 @@ class DecodeGraphs:
         try:
             with torch.cuda.graph(graph, pool=self._pool, capture_error_mode="thread_local"):
                 logits = self._forward(bucket, limit)
+        except Exception:  # noqa: BLE001 - the step itself has run: its result stands, only the graph is lost
+            self._note_failure()
+            return eager
         finally:
             if was_enabled:
                 gc.enable()
-        # capture launches nothing: replay once so that `logits` holds this step's result
-        graph.replay()
+        # Capture launches nothing, and the ordinary run above was this step: its logits are the step's result. The
+        # graph is not replayed on top of it: a step may run once only where a mixer carries a state from token
+        # to token (keys and values written twice land in the same places; a state moved on twice does not).
         bucket.graphs[limit] = (graph, logits)
-        self.replays += 1
-        del eager
-        return logits
+        self.replays += 1                                # steps served here, the one that made the graph included
+        return eager
