@@ -17,6 +17,9 @@ serves it), points at batch 1 and 32, and a cache that takes the card's memory u
 the time to the first token and the time per output token after it, defined as the reference's load
 generator defines them (benchmarks/load/stats.py:29-34, 67-86).
 
+`--design musutar [--size w1024|w2048|w4096]`: prefill and decode of the Musutar decoder beside a Qwen2 decoder of
+equal width, depth, heads and weights, at layer sizes of real models; one JSON line with both for every size.
+
 Random weights N(0, 0.02), seeded uniform token ids.
 """
 
@@ -189,6 +192,82 @@ def serve_run(llm, vocab, seed):
     }
 
 
+# ---- `--design musutar`: the Musutar decoder beside a Qwen2 decoder of equal size, at layer sizes of real models
+# (width, layers, query heads, kv heads, head size, feed-forward, window); vocabulary 32,768, random weights.
+DESIGN_SIZES = {
+    "w1024": dict(width=1024, layers=8, heads=8, kv_heads=2, dim=128, ff=4096, window=1024),
+    "w2048": dict(width=2048, layers=16, heads=16, kv_heads=4, dim=128, ff=8192, window=1024),
+    "w4096": dict(width=4096, layers=8, heads=32, kv_heads=8, dim=128, ff=14336, window=2048),
+}
+DESIGN_VOCAB = 32768
+
+
+def musutar_config(size):
+    """Groups of four layers as the design's own models have them: three windowed attention layers and one state
+    layer; from the second group on the attention layers borrow the keys and values of the first group's last."""
+    z = DESIGN_SIZES[size]
+    rot = {"base": 10000.0, "dims": z["dim"], "scaling": {"factor": 2.0, "original": 2048, "fast": 32.0, "slow": 1.0}}
+    layers = []
+    for i in range(z["layers"]):
+        mlp = {"kind": "dense", "ff": z["ff"]}
+        if i % 4 == 3:
+            decay = [1.0 - 2.0 ** -(2 + 6 * h / max(1, z["heads"] - 1)) for h in range(z["heads"])]
+            layers.append({"type": "lightning", "mlp": mlp,
+                           "mixer": {"heads": z["heads"], "dim": z["dim"], "vdim": z["dim"], "decay": decay}})
+            continue
+        mixer = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "conv": 4,
+                 "mask": {"size": z["window"]}, "rot": rot, "scale": z["dim"] ** -0.5}
+        if i >= 4:
+            mixer["kv_from"] = 2
+        layers.append({"type": "attention", "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Musutar", "vocab": DESIGN_VOCAB, "width": z["width"], "streams": 2, "norm": {"eps": 1e-6},
+            "canon": {"taps": 3}, "layers": layers}
+
+
+def qwen2_equal(size):
+    """The Qwen2 decoder with the same width, depth and heads and a feed-forward sized so that a layer holds as many
+    weights as the Musutar layer (whose gates and projections of the gates count)."""
+    z = DESIGN_SIZES[size]
+    C, q, kv = z["width"], z["heads"] * z["dim"], z["kv_heads"] * z["dim"]
+    musutar_layer = C * (2 * q + 2 * kv) + q * C + 2 * C * C + 2 * C * z["ff"]
+    inter = (musutar_layer - C * (q + 2 * kv) - q * C) // (3 * C) // 32 * 32
+    return dict(COMMON, num_hidden_layers=z["layers"], hidden_size=C, num_attention_heads=z["heads"],
+                num_key_value_heads=z["kv_heads"], head_dim=z["dim"], intermediate_size=inter, vocab_size=DESIGN_VOCAB,
+                rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=8192)
+
+
+def design_run(args) -> int:
+    import torch
+
+    from distie_amd import LLM
+
+    context, prefill_tokens = args.context or 2048, args.prefill or 2048
+    tokens_per_request = context + args.warmup + args.steps + early_tokens(args.batch, context)
+    pages = max(args.batch * -(-tokens_per_request // BLOCK_SIZE), -(-prefill_tokens // BLOCK_SIZE)) + 8
+    sizes = {}
+    for size in ([args.size] if args.size else list(DESIGN_SIZES)):
+        row = {}
+        for name, config in (("musutar", musutar_config(size)), ("qwen2", qwen2_equal(size))):
+            llm = LLM(config=config, random_weights=True, seed=0, dtype=args.dtype, block_size=BLOCK_SIZE,
+                      num_blocks=pages, max_seqs=args.batch, token_budget=TOKEN_BUDGET, use_graphs=True,
+                      max_model_len=max(8192, tokens_per_request), tune_products=not args.no_tune)
+            t_prefill = prefill_run(llm, prefill_tokens, TOKEN_BUDGET, DESIGN_VOCAB)
+            step_s, _ = decode_run(llm, args.batch, context, args.steps, args.warmup, DESIGN_VOCAB, seed=1)
+            row[name] = {"weights_M": round(llm.model.weight_bytes() / (2 if args.dtype == "bf16" else 4) / 1e6, 1),
+                         "prefill_tok_s": round(prefill_tokens / t_prefill, 1), "prefill_ms": round(t_prefill * 1e3, 3),
+                         "decode_tok_s": round(args.batch / step_s, 1), "decode_ms_per_step": round(step_s * 1e3, 4)}
+            llm.close()
+            del llm
+            torch.cuda.empty_cache()
+        sizes[size] = dict(DESIGN_SIZES[size], **row)
+    print(json.dumps({"metric": "prefill and decode tok/s, Musutar beside Qwen2 at equal size", "unit": "tok/s",
+                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype, "data": "synthetic",
+                      "config": {"batch": args.batch, "context": context, "prefill_tokens": prefill_tokens,
+                                 "vocab": DESIGN_VOCAB, "block_size": BLOCK_SIZE, "captured_decode": True},
+                      "sizes": sizes}), flush=True)
+    return 0
+
+
 def main() -> int:
     parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     parser.add_argument("--gpus", type=int, default=1)
@@ -212,10 +291,15 @@ def main() -> int:
                         help="size the cache from free memory (the default for --shape 32b and --serve: 0.9)")
     parser.add_argument("--packed-weights", default=None, metavar="ROLES",
                         help="packed copies only for these products (qkv,attn_out,gate_up,down,head); 'none' for no copies")
+    parser.add_argument("--design", default=None, choices=["musutar"],
+                        help="instead of the workload above: this design beside a Qwen2 decoder of equal size, prefill and decode")
+    parser.add_argument("--size", default=None, choices=sorted(DESIGN_SIZES), help="with --design: one size instead of all")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported (this engine has no multi-GPU path)")
         return 2
+    if args.design:
+        return design_run(args)
 
     import torch
 

@@ -41,7 +41,7 @@ from ..config.model_config import PartSpec
 @dataclass(frozen=True)
 class ParamSpec:
     shape: Tuple[int, ...]
-    init: str = "normal"   # "normal" | "ones" | "zeros" | "int"
+    init: str = "normal"   # "normal" | "ones" | "zeros" | "int" | "eye" (a square matrix: the identity)
 
 
 PAGE = -1      # stands for the page size in the shape of a paged tensor

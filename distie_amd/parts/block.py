@@ -66,7 +66,7 @@ class HyperConnections(Block):
         for q in self.subs:
             if self.streams is not None:
                 specs.update({f"hc{q}.in": ParamSpec((S,), "ones"), f"hc{q}.out": ParamSpec((S,), "ones"),
-                              f"hc{q}.mix": ParamSpec((S, S))})
+                              f"hc{q}.mix": ParamSpec((S, S), "eye")})
         if self.input_taps:
             specs["canon1"] = ParamSpec((C, self.input_taps))
         for q in self.subs:

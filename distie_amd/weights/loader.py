@@ -94,6 +94,8 @@ def random_tensor(name: str, spec, seed: int, std: float, device) -> torch.Tenso
         return torch.zeros(spec.shape, dtype=torch.float32, device=device)
     if spec.init == "int":
         return torch.zeros(spec.shape, dtype=torch.int32, device=device)
+    if spec.init == "eye":
+        return torch.eye(spec.shape[0], spec.shape[1], dtype=torch.float32, device=device)
     count = 1
     for n in spec.shape:
         count *= int(n)
