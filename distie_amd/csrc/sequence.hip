@@ -23,9 +23,11 @@ __device__ __forceinline__ float siluf(float x) { return x / (1.f + __expf(-x));
 //   write:  x_j <- sum_s mix[s, j] x_s + out_w[j] * y * sigmoid(gate)   (all streams at once from the old ones)
 //   read:   u = sum_s in_w[s] x_s;  h = norm(u) * weight                (kind 0: u itself, 1: centred, 2: root mean square)
 // One block a token; u of the whole row waits in LDS between the two passes of the statistics.
-template <typename Y, typename G, typename W, typename H>
+// MS: the most streams this instance takes (its loops are unrolled to that, so the streams stay in registers).
+template <int MS, typename Y, typename G, typename W, typename H>
 __global__ void hyper_step_kernel(float* __restrict__ streams, int S, const float* __restrict__ init, const Y* __restrict__ y,
                                   int y_slices, int64_t y_slice_stride, const G* __restrict__ gate, int64_t gate_ld,
+                                  int gate_slices, int64_t gate_slice_stride,
                                   const float* __restrict__ mix, const float* __restrict__ out_w,
                                   const float* __restrict__ in_w, const W* __restrict__ norm_w, int kind, float eps,
                                   H* __restrict__ h, int C) {
@@ -33,38 +35,48 @@ __global__ void hyper_step_kernel(float* __restrict__ streams, int S, const floa
   __shared__ float scratch[16];
   const int64_t t = blockIdx.x;
   float* x = streams + t * S * C;
-  float m[MAX_STREAMS * MAX_STREAMS], ow[MAX_STREAMS], iw[MAX_STREAMS];
-  if (y != nullptr) {
-    for (int i = 0; i < S * S; ++i) m[i] = mix[i];
-    for (int i = 0; i < S; ++i) ow[i] = out_w[i];
+  float m[MS][MS], ow[MS], iw[MS];
+#pragma unroll
+  for (int i = 0; i < MS; ++i) {
+    ow[i] = (y != nullptr && i < S) ? out_w[i] : 0.f;
+    iw[i] = (h != nullptr && i < S) ? in_w[i] : 0.f;
+#pragma unroll
+    for (int j = 0; j < MS; ++j) m[i][j] = (y != nullptr && i < S && j < S) ? mix[i * S + j] : 0.f;
   }
-  if (h != nullptr)
-    for (int i = 0; i < S; ++i) iw[i] = in_w[i];
   float sum = 0.f;
   for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float v[MAX_STREAMS];
+    float v[MS];
     if (init != nullptr) {
       const float e = init[t * C + c];
-      for (int s = 0; s < S; ++s) v[s] = e;
+#pragma unroll
+      for (int s = 0; s < MS; ++s) v[s] = s < S ? e : 0.f;
     } else {
-      for (int s = 0; s < S; ++s) v[s] = x[s * C + c];
+#pragma unroll
+      for (int s = 0; s < MS; ++s) v[s] = s < S ? x[s * C + c] : 0.f;
     }
     if (y != nullptr) {
       float d = sum_strided(y + t * C + c, y_slices, y_slice_stride);
-      if (gate != nullptr) d *= sigmoidf(to_float(gate[t * gate_ld + c]));
-      float n[MAX_STREAMS];
-      for (int j = 0; j < S; ++j) {
+      if (gate != nullptr) d *= sigmoidf(sum_strided(gate + t * gate_ld + c, gate_slices, gate_slice_stride));
+      float n[MS];
+#pragma unroll
+      for (int j = 0; j < MS; ++j) {
         float a = 0.f;
-        for (int s = 0; s < S; ++s) a += m[s * S + j] * v[s];
+#pragma unroll
+        for (int s = 0; s < MS; ++s) a += m[s][j] * v[s];
         n[j] = a + ow[j] * d;
       }
-      for (int j = 0; j < S; ++j) v[j] = n[j];
+#pragma unroll
+      for (int j = 0; j < MS; ++j) v[j] = n[j];
     }
-    if (init != nullptr || y != nullptr)
-      for (int s = 0; s < S; ++s) x[s * C + c] = v[s];
+    if (init != nullptr || y != nullptr) {
+#pragma unroll
+      for (int s = 0; s < MS; ++s)
+        if (s < S) x[s * C + c] = v[s];
+    }
     if (h != nullptr) {
       float u = 0.f;
-      for (int s = 0; s < S; ++s) u += iw[s] * v[s];
+#pragma unroll
+      for (int s = 0; s < MS; ++s) u += iw[s] * v[s];
       row[c] = u;
       sum += kind == 2 ? u * u : u;
     }
@@ -165,35 +177,56 @@ __global__ void conv_state_kernel(const X* __restrict__ x, int64_t ldx, int taps
 // and sine from `table` [T, pairs, 2], both times `magnitude`); q goes to q_out [T, H, DP] (zeros beyond D), k
 // and v to the token's slot of the cache, k [pages, G, P, DP], v [pages, G, DP, P] (what lies beyond D and E there
 // was zero when the cache was made and is never written).
+// One block a (token, head): q heads, then k heads, then v heads. A thread owns its channels alone, so for a request
+// that brings one row it also moves the convolution's state on (`conv_state_kernel` does it for the others).
 template <typename X, typename W, typename Q, typename C>
 __global__ void conv_rope_kv_write_kernel(const X* __restrict__ product, int64_t ld, const W* __restrict__ weight, int taps,
-                                          const float* __restrict__ state, const float2* __restrict__ table, int pairs,
+                                          float* __restrict__ state, const float2* __restrict__ table, int pairs,
                                           float magnitude, Q* __restrict__ q_out, C* __restrict__ k_cache,
                                           C* __restrict__ v_cache, const int32_t* __restrict__ slots,
                                           const int32_t* __restrict__ cu_q, const int32_t* __restrict__ token_request,
                                           const int32_t* __restrict__ state_slots, int H, int G, int D, int E, int DP,
                                           int block_size, int has_kv, int write) {
   const int64_t t = blockIdx.x;
+  const int head = blockIdx.y;
   const int N = H * D + (has_kv ? G * (D + E) : 0);
   const int b = token_request[t];
-  const int i = static_cast<int>(t) - cu_q[b];
-  const float* own = taps > 1 ? state + static_cast<int64_t>(state_slots[b]) * (taps - 1) * N : nullptr;
+  const int first = cu_q[b];
+  const int i = static_cast<int>(t) - first;
+  const bool single = cu_q[b + 1] - first == 1;
+  float* own = taps > 1 ? state + static_cast<int64_t>(state_slots[b]) * (taps - 1) * N : nullptr;
   const int64_t slot = (has_kv && write) ? slots[t] : 0;
   const int64_t page = slot / block_size;
   const int offset = static_cast<int>(slot % block_size);
   auto value = [&](int c) {
-    if (taps < 1) return to_float(product[t * ld + c]);
+    const float self = to_float(product[t * ld + c]);
+    if (taps < 1) return self;
     float w[MAX_TAPS];
     for (int j = 0; j < taps; ++j) w[j] = to_float(weight[static_cast<int64_t>(c) * taps + j]);
-    return conv_at(product, ld, own, w, taps, t, i, c, N);
+    const float acc = conv_at(product, ld, own, w, taps, t, i, c, N);
+    if (single && taps > 1) {
+      float keep[MAX_TAPS];
+      for (int k = 1; k < taps - 1; ++k) keep[k] = own[static_cast<int64_t>(k) * N + c];
+      for (int k = 1; k < taps - 1; ++k) own[static_cast<int64_t>(k - 1) * N + c] = keep[k];
+      own[static_cast<int64_t>(taps - 2) * N + c] = self;
+    }
+    return acc;
   };
-  // q and k: a thread owns a pair, or a single dimension beyond the turned ones; (H + G) heads of DP places
-  const int turned = has_kv ? H + G : H;
-  const int per_head = DP - pairs;                       // pairs count once
-  for (int item = threadIdx.x; item < turned * per_head; item += blockDim.x) {
-    const int head = item / per_head;
-    const int j = item % per_head;
-    const int base = head * D;                           // q heads, then k heads: both D wide, one after the other
+  if (head >= H + G) {                                   // a v head
+    if (!write) {
+      if (single && taps > 1)
+        for (int e = threadIdx.x; e < E; e += blockDim.x) (void)value((H + G) * D + (head - H - G) * E + e);
+      return;
+    }
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+      const float v = value((H + G) * D + (head - H - G) * E + e);
+      v_cache[((page * G + (head - H - G)) * DP + e) * block_size + offset] = from_float<C>(to_float(from_float<Q>(v)));
+    }
+    return;
+  }
+  // q and k: a thread owns a pair, or a single dimension beyond the turned ones
+  const int base = head * D;                             // q heads, then k heads: both D wide, one after the other
+  for (int j = threadIdx.x; j < DP - pairs; j += blockDim.x) {
     float a, bq = 0.f;
     int d0, d1 = -1;
     if (j < pairs) {
@@ -217,13 +250,6 @@ __global__ void conv_rope_kv_write_kernel(const X* __restrict__ product, int64_t
       k[d0] = from_float<C>(to_float(from_float<Q>(a)));
       if (d1 >= 0) k[d1] = from_float<C>(to_float(from_float<Q>(bq)));
     }
-  }
-  if (!has_kv || !write) return;
-  for (int item = threadIdx.x; item < G * E; item += blockDim.x) {
-    const int head = item / E;
-    const int e = item % E;
-    const float v = value((H + G) * D + item);
-    v_cache[((page * G + head) * DP + e) * block_size + offset] = from_float<C>(to_float(from_float<Q>(v)));
   }
 }
 
@@ -259,12 +285,12 @@ __global__ void rmsnorm_gate_kernel(const float* __restrict__ x, const W* __rest
 }
 
 // kinds: 0 relu squared, 1 silu, 2 gelu (tanh form), 3 relu
-template <typename T>
-__global__ void activation_kernel(const T* __restrict__ in, int slices, int64_t slice_stride, T* __restrict__ out,
+template <typename I, typename T>
+__global__ void activation_kernel(const I* __restrict__ in, int slices, int64_t slice_stride, T* __restrict__ out,
                                   int64_t count, int kind) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= count) return;
-  const float z = slices == 1 ? to_float(in[i]) : 0.f;
+  const float z = sum_strided(in + i, slices, slice_stride);
   float r;
   if (kind == 0) {
     const float p = fmaxf(z, 0.f);
@@ -338,17 +364,222 @@ decay_scan_kernel(const X* __restrict__ product, int64_t ld, float* __restrict__
   }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// The same recurrence over portions of prompts, in chunks of 64 rows that run side by side. With L the rows of a
+// chunk, S the state in front of it and w^m the decay's powers (a table made by repeated multiplication):
+//   sums:     P[d][e]   = sum_j w^(L-1-j) k_j[d] v_j[e]                      (each chunk alone)
+//   states:   S_next    = w^L S + P, chunk after chunk; S (the state in front) takes P's place in the scratch
+//   outputs:  o_i[e]    = w^(i+1) sum_d q_i[d] S[d][e] + sum_{j<=i} w^(i-j) (q_i . k_j) v_j[e]
+// Only non-negative powers occur, so nothing grows with the chunk's length. Float32 throughout, FMAs on tiles
+// held in LDS; a chunk's table entry is {request, first row, rows, unused}.
+constexpr int SCAN_L = 64;
+constexpr int SCAN_PAD = 68;      // row stride of the transposed tiles: keeps 16-byte reads aligned
+
+__device__ __forceinline__ void decay_powers(float* pw, float rate, int count) {
+  if (threadIdx.x == 0) {
+    float p = 1.f;
+    for (int m = 0; m < count; ++m) {
+      pw[m] = p;
+      p *= rate;
+    }
+  }
+}
+
+template <typename X>
+__global__ void __launch_bounds__(256)
+scan_chunk_sums_kernel(const X* __restrict__ product, int64_t ld, const float* __restrict__ decay, float* __restrict__ scratch,
+                       const int4* __restrict__ chunks, int H, int D, int E) {
+  extern __shared__ float lds[];
+  float* Ks = lds;                       // [64][D], each row times its power of the decay
+  float* Vs = Ks + SCAN_L * D;           // [64][64]
+  float* pw = Vs + SCAN_L * 64;          // [65]
+  const int c = blockIdx.x, head = blockIdx.y, e0 = blockIdx.z * 64;
+  const int4 chunk = chunks[c];
+  const int64_t row0 = chunk.y;
+  const int len = chunk.z;
+  decay_powers(pw, decay[head], SCAN_L + 1);
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < SCAN_L * D; idx += 256) {
+    const int j = idx / D, d = idx % D;
+    Ks[idx] = j < len ? pw[len - 1 - j] * siluf(to_float(product[(row0 + j) * ld + (H + head) * D + d])) : 0.f;
+  }
+  for (int idx = threadIdx.x; idx < SCAN_L * 64; idx += 256) {
+    const int j = idx / 64, e = e0 + idx % 64;
+    Vs[idx] = (j < len && e < E) ? siluf(to_float(product[(row0 + j) * ld + 2 * H * D + head * E + e])) : 0.f;
+  }
+  __syncthreads();
+  const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+  float acc[2][4][4] = {};
+  for (int j = 0; j < len; ++j) {
+    const float4 v4 = *reinterpret_cast<const float4*>(Vs + j * 64 + 4 * tx);
+    const float v[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int d0 = 4 * ty + 64 * s;
+      if (d0 >= D) break;
+      const float4 k4 = *reinterpret_cast<const float4*>(Ks + j * D + d0);
+      const float k[4] = {k4.x, k4.y, k4.z, k4.w};
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[s][a][b] += k[a] * v[b];
+    }
+  }
+  float* dst = scratch + (static_cast<int64_t>(c) * H + head) * D * E;
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int d = 4 * ty + 64 * s + a;
+      if (d >= D) continue;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int e = e0 + 4 * tx + b;
+        if (e < E) dst[static_cast<int64_t>(d) * E + e] = acc[s][a][b];
+      }
+    }
+}
+
+__global__ void scan_chunk_states_kernel(float* __restrict__ scratch, float* __restrict__ state, const float* __restrict__ decay,
+                                         const int4* __restrict__ chunks, const int32_t* __restrict__ request_chunks,
+                                         const int32_t* __restrict__ state_slots, int H, int D, int E) {
+  const int b = blockIdx.x, head = blockIdx.y;
+  const int idx = blockIdx.z * blockDim.x + threadIdx.x;
+  if (idx >= D * E) return;
+  const int c0 = request_chunks[b], c1 = request_chunks[b + 1];
+  if (c0 >= c1) return;
+  const float rate = decay[head];
+  float full = 1.f;
+  for (int m = 0; m < SCAN_L; ++m) full *= rate;
+  float* own = state + (static_cast<int64_t>(state_slots[b]) * H + head) * D * E + idx;
+  const int64_t stride = static_cast<int64_t>(H) * D * E;
+  float* p = scratch + (static_cast<int64_t>(c0) * H + head) * D * E + idx;
+  float S = *own;
+  for (int c = c0; c < c1; c += 4) {
+    // the sums of four chunks are asked for together; each then gives way to the state in front of its chunk
+    float add[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) add[u] = c + u < c1 ? p[u * stride] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (c + u >= c1) break;
+      const int len = chunks[c + u].z;
+      float f = full;
+      if (len != SCAN_L) {
+        f = 1.f;
+        for (int m = 0; m < len; ++m) f *= rate;
+      }
+      p[u * stride] = S;
+      S = f * S + add[u];
+    }
+    p += 4 * stride;
+  }
+  *own = S;
+}
+
+template <typename X>
+__global__ void __launch_bounds__(256)
+scan_chunk_outputs_kernel(const X* __restrict__ product, int64_t ld, const float* __restrict__ decay,
+                          const float* __restrict__ scratch, float* __restrict__ out, const int4* __restrict__ chunks,
+                          int H, int D, int E) {
+  extern __shared__ float lds[];
+  float* Qt = lds;                       // [D][68]: Qt[d][i]
+  float* Kt = Qt + D * SCAN_PAD;         // [D][68]; once the scores are made, the state in front of the chunk [D][64]
+  float* At = Kt + D * SCAN_PAD;         // [64][68]: At[j][i] = w^(i-j) q_i . k_j for j <= i
+  float* Vs = At + SCAN_L * SCAN_PAD;    // [64][64]
+  float* pw = Vs + SCAN_L * 64;          // [66]
+  const int c = blockIdx.x, head = blockIdx.y, e0 = blockIdx.z * 64;
+  const int4 chunk = chunks[c];
+  const int64_t row0 = chunk.y;
+  const int len = chunk.z;
+  decay_powers(pw, decay[head], SCAN_L + 2);
+  for (int idx = threadIdx.x; idx < SCAN_L * D; idx += 256) {
+    const int j = idx / D, d = idx % D;
+    float q = 0.f, k = 0.f;
+    if (j < len) {
+      const X* row = product + (row0 + j) * ld;
+      q = siluf(to_float(row[head * D + d]));
+      k = siluf(to_float(row[(H + head) * D + d]));
+    }
+    Qt[d * SCAN_PAD + j] = q;
+    Kt[d * SCAN_PAD + j] = k;
+  }
+  for (int idx = threadIdx.x; idx < SCAN_L * 64; idx += 256) {
+    const int j = idx / 64, e = e0 + idx % 64;
+    Vs[idx] = (j < len && e < E) ? siluf(to_float(product[(row0 + j) * ld + 2 * H * D + head * E + e])) : 0.f;
+  }
+  __syncthreads();
+  const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+  float s4[4][4] = {};
+  if (tx <= ty) {
+    for (int d = 0; d < D; ++d) {
+      const float4 q4 = *reinterpret_cast<const float4*>(Qt + d * SCAN_PAD + 4 * ty);
+      const float4 k4 = *reinterpret_cast<const float4*>(Kt + d * SCAN_PAD + 4 * tx);
+      const float q[4] = {q4.x, q4.y, q4.z, q4.w}, k[4] = {k4.x, k4.y, k4.z, k4.w};
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) s4[a][b] += q[a] * k[b];
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int i = 4 * ty + a, j = 4 * tx + b;
+      At[j * SCAN_PAD + i] = j <= i ? pw[i - j] * s4[a][b] : 0.f;
+    }
+  __syncthreads();
+  float* Ss = Kt;
+  const float* src = scratch + (static_cast<int64_t>(c) * H + head) * D * E;
+  for (int idx = threadIdx.x; idx < D * 64; idx += 256) {
+    const int d = idx / 64, e = e0 + idx % 64;
+    Ss[idx] = e < E ? src[static_cast<int64_t>(d) * E + e] : 0.f;
+  }
+  __syncthreads();
+  float o[4][4] = {}, r[4][4] = {};
+  for (int d = 0; d < D; ++d) {
+    const float4 q4 = *reinterpret_cast<const float4*>(Qt + d * SCAN_PAD + 4 * ty);
+    const float4 t4 = *reinterpret_cast<const float4*>(Ss + d * 64 + 4 * tx);
+    const float q[4] = {q4.x, q4.y, q4.z, q4.w}, t[4] = {t4.x, t4.y, t4.z, t4.w};
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) r[a][b] += q[a] * t[b];
+  }
+  const int reach = min(len, 4 * ty + 4);
+  for (int j = 0; j < reach; ++j) {
+    const float4 a4 = *reinterpret_cast<const float4*>(At + j * SCAN_PAD + 4 * ty);
+    const float4 v4 = *reinterpret_cast<const float4*>(Vs + j * 64 + 4 * tx);
+    const float w[4] = {a4.x, a4.y, a4.z, a4.w}, v[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) o[a][b] += w[a] * v[b];
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int i = 4 * ty + a;
+    if (i >= len) continue;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int e = e0 + 4 * tx + b;
+      if (e < E) out[((row0 + i) * H + head) * E + e] = o[a][b] + pw[i + 1] * r[a][b];
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" int distie_hyper_step(float* streams, int S, const float* init, const void* y, int y_dtype, int y_slices,
-                                 const void* gate, int gate_dtype, int64_t gate_ld, const float* mix, const float* out_w,
+                                 const void* gate, int gate_dtype, int64_t gate_ld, int gate_slices, const float* mix,
+                                 const float* out_w,
                                  const float* in_w, const void* norm_w, int norm_dtype, int kind, float eps, void* h,
                                  int h_dtype, int T, int C, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (S < 1 || S > MAX_STREAMS || C < 1 || kind < 0 || kind > 2 || y_slices < 1) return DISTIE_BAD_ARGUMENT;
+  if (S < 1 || S > MAX_STREAMS || C < 1 || kind < 0 || kind > 2 || y_slices < 1 || gate_slices < 1) return DISTIE_BAD_ARGUMENT;
   if (y != nullptr && (mix == nullptr || out_w == nullptr)) return DISTIE_BAD_ARGUMENT;
   if (h != nullptr && (in_w == nullptr || (kind != 0 && norm_w == nullptr))) return DISTIE_BAD_ARGUMENT;
-  if (static_cast<size_t>(C) * sizeof(float) > 64 * 1024) return DISTIE_BAD_ARGUMENT;
   const int threads = C >= 2048 ? 512 : (C >= 512 ? 256 : (C >= 128 ? 128 : 64));
   const size_t lds = h != nullptr ? static_cast<size_t>(C) * sizeof(float) : 0;
   const int64_t y_stride = static_cast<int64_t>(T) * C;
@@ -356,10 +587,22 @@ extern "C" int distie_hyper_step(float* streams, int S, const float* init, const
   if (gate == nullptr) gate_dtype = y_dtype;
   if (norm_w == nullptr) norm_dtype = DISTIE_F32;
   if (h == nullptr) h_dtype = DISTIE_F32;
-  DISTIE_DISPATCH(y_dtype, Y, DISTIE_DISPATCH(gate_dtype, G, DISTIE_DISPATCH(norm_dtype, W, DISTIE_DISPATCH(h_dtype, HT,
-      hyper_step_kernel<Y, G, W, HT><<<T, threads, lds, stream>>>(
-          streams, S, init, static_cast<const Y*>(y), y_slices, y_stride, static_cast<const G*>(gate), gate_ld, mix, out_w,
-          in_w, static_cast<const W*>(norm_w), kind, eps, static_cast<HT*>(h), C)))));
+  if (lds > 48 * 1024) return DISTIE_BAD_ARGUMENT;      // a row of u waits in LDS: widths up to 12,288
+#define DISTIE_HYPER(MS)                                                                                               \
+  DISTIE_DISPATCH(y_dtype, Y, DISTIE_DISPATCH(gate_dtype, G, DISTIE_DISPATCH(norm_dtype, W, DISTIE_DISPATCH(h_dtype, HT,  \
+      hyper_step_kernel<MS, Y, G, W, HT><<<T, threads, lds, stream>>>(                                                \
+          streams, S, init, static_cast<const Y*>(y), y_slices, y_stride, static_cast<const G*>(gate), gate_ld,       \
+          gate_slices, gate_ld * T, mix, out_w, in_w, static_cast<const W*>(norm_w), kind, eps, static_cast<HT*>(h), C)))))
+  if (S == 1) {
+    DISTIE_HYPER(1);
+  } else if (S == 2) {
+    DISTIE_HYPER(2);
+  } else if (S <= 4) {
+    DISTIE_HYPER(4);
+  } else {
+    DISTIE_HYPER(8);
+  }
+#undef DISTIE_HYPER
   return launch_status();
 }
 
@@ -390,7 +633,7 @@ extern "C" int distie_conv_state(const void* x, int x_dtype, int64_t ldx, int ta
 }
 
 extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t ld, const void* weight, int w_dtype,
-                                         int taps, const float* state, const void* table, int pairs, float magnitude,
+                                         int taps, float* state, const void* table, int pairs, float magnitude,
                                          void* q_out, void* k_cache, void* v_cache, int cache_dtype, const int32_t* slots,
                                          const int32_t* cu_q, const int32_t* token_request, const int32_t* state_slots,
                                          int T, int H, int G, int D, int E, int DP, int block_size, int has_kv, int write,
@@ -402,11 +645,12 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
   if ((pairs > 0 && table == nullptr) || (taps > 1 && state == nullptr) || (taps >= 1 && weight == nullptr))
     return DISTIE_BAD_ARGUMENT;
   if (has_kv && write && (k_cache == nullptr || v_cache == nullptr || slots == nullptr)) return DISTIE_BAD_ARGUMENT;
-  const int work = (H + G) * DP;
-  const int threads = work >= 1024 ? 256 : (work >= 256 ? 128 : 64);
+  const int work = DP - pairs > E ? DP - pairs : E;
+  const int threads = work > 128 ? 256 : (work > 64 ? 128 : 64);
+  const dim3 grid(T, has_kv ? H + 2 * G : H);
   if (weight == nullptr) w_dtype = dtype;
   DISTIE_DISPATCH(dtype, X, DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(cache_dtype, C,
-      conv_rope_kv_write_kernel<X, W, X, C><<<T, threads, 0, stream>>>(
+      conv_rope_kv_write_kernel<X, W, X, C><<<grid, threads, 0, stream>>>(
           static_cast<const X*>(product), ld, static_cast<const W*>(weight), taps, state, static_cast<const float2*>(table),
           pairs, magnitude, static_cast<X*>(q_out), static_cast<C*>(k_cache), static_cast<C*>(v_cache), slots, cu_q,
           token_request, state_slots, H, G, D, E, DP, block_size, has_kv, write))));
@@ -437,14 +681,16 @@ extern "C" int distie_rmsnorm_gate(const float* x, const void* weight, int w_dty
   return launch_status();
 }
 
-extern "C" int distie_activation(const void* in, void* out, int dtype, int64_t count, int kind, hipStream_t stream) {
+extern "C" int distie_activation(const void* in, int in_dtype, int slices, void* out, int dtype, int64_t count, int kind,
+                                 hipStream_t stream) {
   if (count <= 0) return 0;
-  if (kind < 0 || kind > 3) return DISTIE_BAD_ARGUMENT;
+  if (kind < 0 || kind > 3 || slices < 1) return DISTIE_BAD_ARGUMENT;
   const int threads = 256;
   const int64_t blocks = (count + threads - 1) / threads;
   if (blocks > 0x7fffffff) return DISTIE_BAD_ARGUMENT;
-  DISTIE_DISPATCH(dtype, T, activation_kernel<T><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(
-      static_cast<const T*>(in), 1, 0, static_cast<T*>(out), count, kind));
+  DISTIE_DISPATCH(in_dtype, I, DISTIE_DISPATCH(dtype, T,
+      activation_kernel<I, T><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(
+          static_cast<const I*>(in), slices, count, static_cast<T*>(out), count, kind)));
   return launch_status();
 }
 
@@ -470,5 +716,46 @@ extern "C" int distie_decay_scan(const void* product, int dtype, int64_t ld, flo
     DISTIE_SCAN(8, 32);
   }
 #undef DISTIE_SCAN
+  return launch_status();
+}
+
+// rows of a chunk, and the largest key size the chunked scan takes (its tiles must fit the LDS)
+extern "C" int distie_decay_scan_chunk_rows() { return SCAN_L; }
+extern "C" int distie_decay_scan_chunked_max_dim() { return 128; }
+
+template <typename K>
+static int more_lds(K kernel, size_t lds) {
+  if (lds <= 48 * 1024) return 0;
+  return static_cast<int>(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              static_cast<int>(lds)));
+}
+
+// chunks: int32 [num_chunks][4] = {request, first row, rows (1..64), 0}, the chunks of a request one after the other;
+// request_chunks: int32 [B + 1], the first chunk of every request; scratch: float32 [num_chunks, H, D, E]
+extern "C" int distie_decay_scan_chunked(const void* product, int dtype, int64_t ld, float* state, const float* decay,
+                                         float* out, float* scratch, const int32_t* chunks, const int32_t* request_chunks,
+                                         const int32_t* state_slots, int num_chunks, int B, int H, int D, int E,
+                                         hipStream_t stream) {
+  if (B <= 0 || num_chunks <= 0) return 0;
+  if (H < 1 || D < 4 || E < 4 || D % 4 || E % 4 || D > 128 || ld < static_cast<int64_t>(H) * (2 * D + E))
+    return DISTIE_BAD_ARGUMENT;
+  const dim3 grid(num_chunks, H, (E + 63) / 64);
+  const int4* table = reinterpret_cast<const int4*>(chunks);
+  const size_t lds_sums = (static_cast<size_t>(SCAN_L) * D + SCAN_L * 64 + SCAN_L + 1) * sizeof(float);
+  const size_t lds_out = (2 * static_cast<size_t>(D) * SCAN_PAD + SCAN_L * SCAN_PAD + SCAN_L * 64 + SCAN_L + 2) * sizeof(float);
+  int status = 0;
+  DISTIE_DISPATCH(dtype, X, {
+    if ((status = more_lds(scan_chunk_sums_kernel<X>, lds_sums)) != 0) return status;
+    scan_chunk_sums_kernel<X><<<grid, 256, lds_sums, stream>>>(static_cast<const X*>(product), ld, decay, scratch, table, H, D, E);
+  });
+  if ((status = launch_status()) != 0) return status;
+  scan_chunk_states_kernel<<<dim3(B, H, (D * E + 255) / 256), 256, 0, stream>>>(scratch, state, decay, table, request_chunks,
+                                                                               state_slots, H, D, E);
+  if ((status = launch_status()) != 0) return status;
+  DISTIE_DISPATCH(dtype, X, {
+    if ((status = more_lds(scan_chunk_outputs_kernel<X>, lds_out)) != 0) return status;
+    scan_chunk_outputs_kernel<X><<<grid, 256, lds_out, stream>>>(static_cast<const X*>(product), ld, decay, scratch, out, table,
+                                                                H, D, E);
+  });
   return launch_status();
 }

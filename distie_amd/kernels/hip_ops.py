@@ -292,15 +292,16 @@ class HipOps(Ops):
         o.distie_decode_product_residual.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
         o.distie_decode_norm_product.argtypes = [_P, _P, _F, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P,
                                                  _I, _I, _I, _I, _I, _P]
-        o.distie_hyper_step.argtypes = [_P, _I, _P, _P, _I, _I, _P, _I, _L, _P, _P, _P, _P, _I, _I, _F, _P, _I, _I, _I, _P]
+        o.distie_hyper_step.argtypes = [_P, _I, _P, _P, _I, _I, _P, _I, _L, _I, _P, _P, _P, _P, _I, _I, _F, _P, _I, _I, _I, _P]
         o.distie_causal_conv.argtypes = [_P, _I, _L, _P, _I, _I, _P, _P, _I, _L, _I, _P, _P, _P, _I, _I, _P]
         o.distie_conv_state.argtypes = [_P, _I, _L, _I, _P, _P, _P, _I, _I, _I, _P]
         o.distie_conv_rope_kv_write.argtypes = [_P, _I, _L, _P, _I, _I, _P, _P, _I, _F, _P, _P, _P, _I, _P, _P, _P, _P,
                                                 _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]
         o.distie_sigmoid_gate.argtypes = [_P, _I, _I, _I, _P, _I, _L, _P, _I, _I, _I, _P]
         o.distie_rmsnorm_gate.argtypes = [_P, _P, _I, _F, _P, _I, _L, _P, _I, _I, _I, _P]
-        o.distie_activation.argtypes = [_P, _P, _I, _L, _I, _P]
+        o.distie_activation.argtypes = [_P, _I, _I, _P, _I, _L, _I, _P]
         o.distie_decay_scan.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]
+        o.distie_decay_scan_chunked.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
         o.distie_argmax.argtypes = [_P, _P, _I, _I, _P, _P, _P]
         o.distie_argmax_parts.argtypes = [_I, _I]
         o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P]
@@ -1014,6 +1015,9 @@ class HipOps(Ops):
         return t.data_ptr(), t.stride(0)
 
     NORM_KINDS = {"none": 0, "layer": 1, "rms": 2}
+    # a step in which some request brings at least so many rows runs the decayed state in chunks of rows that are
+    # worked side by side (three kernels) instead of row after row (one)
+    SCAN_CHUNKED_MIN_ROWS = 16
     ACTIVATIONS = {"relu2": 0, "silu": 1, "gelu_tanh": 2, "relu": 3}
 
     def hyper_step(self, streams, *, init=None, delta=None, gate=None, mix=None, write=None, read=None,
@@ -1037,7 +1041,7 @@ class HipOps(Ops):
                 raise KernelError(f"hyper_step: {name} must be float32 {list(shape)}")
         if init is not None and tuple(init.shape) != (T, C):
             raise KernelError("hyper_step: init does not match the streams")
-        slices, y, y_code, g_ptr, g_code, g_ld = 1, None, _F32, None, _F32, 0
+        slices, y, y_code, g_ptr, g_code, g_ld, g_slices = 1, None, _F32, None, _F32, 0, 1
         if delta is not None:
             if mix is None or write is None:
                 raise KernelError("hyper_step: a delta needs mix and write weights")
@@ -1050,7 +1054,16 @@ class HipOps(Ops):
                 raise KernelError("hyper_step: delta must be [T, C]")
             y, y_code = delta.data_ptr(), _code(delta)
             if gate is not None:
-                g_ptr, g_ld = self._rows_view(gate, C)
+                if isinstance(gate, (PendingNorm, PendingProduct)):
+                    gate = self.dense(gate)
+                if isinstance(gate, PartialSums):
+                    g_slices, gate = gate.slices, gate.data
+                    self._own(gate)
+                    if tuple(gate.shape[-2:]) != (T, C):
+                        raise KernelError("hyper_step: the gate must be [T, C]")
+                    g_ptr, g_ld = gate.data_ptr(), C
+                else:
+                    g_ptr, g_ld = self._rows_view(gate, C)
                 g_code = _code(gate)
         h = None
         if read is not None:
@@ -1059,7 +1072,7 @@ class HipOps(Ops):
             h = torch.empty((T, C), dtype=out_dtype or torch.float32, device=self.device)
         ptr = lambda t: t.data_ptr() if t is not None else None
         _check(self._ops.distie_hyper_step(
-            streams.data_ptr(), S, ptr(init), y, y_code, slices, g_ptr, g_code, g_ld, ptr(mix), ptr(write), ptr(read),
+            streams.data_ptr(), S, ptr(init), y, y_code, slices, g_ptr, g_code, g_ld, g_slices, ptr(mix), ptr(write), ptr(read),
             ptr(norm_weight), _code(norm_weight) if norm_weight is not None else _F32, self.NORM_KINDS[norm], float(eps),
             ptr(h), _code(h) if h is not None else _F32, T, C, self._stream()), "hyper_step")
         _mark_written(streams)
@@ -1122,9 +1135,11 @@ class HipOps(Ops):
             meta.state_slots.data_ptr(), T, num_heads, num_kv_heads, dim, value_dim, padded_dim, meta.block_size,
             1 if has_kv else 0, 1 if write else 0, self._stream()), "conv_rope_kv_write")
         if taps > 1:
-            _check(self._ops.distie_conv_state(product.data_ptr(), _code(product), W, taps, state.data_ptr(),
-                                               meta.cu_q.data_ptr(), meta.state_slots.data_ptr(), meta.num_requests,
-                                               channels, 0, self._stream()), "conv_state")
+            if not meta.all_decode:
+                # (requests that bring one row had their state moved on by the kernel above)
+                _check(self._ops.distie_conv_state(product.data_ptr(), _code(product), W, taps, state.data_ptr(),
+                                                   meta.cu_q.data_ptr(), meta.state_slots.data_ptr(), meta.num_requests,
+                                                   channels, 1, self._stream()), "conv_state")
             _mark_written(state)
         return q
 
@@ -1152,6 +1167,31 @@ class HipOps(Ops):
         if decay.dtype != torch.float32 or tuple(decay.shape) != (num_heads,):
             raise KernelError("decay_scan: decay must be float32 [heads]")
         out = torch.empty((T, num_heads * value_dim), dtype=torch.float32, device=self.device)
+        if not self.captured and meta.host_cu_q is not None and meta.max_q >= self.SCAN_CHUNKED_MIN_ROWS and \
+                dim % 4 == 0 and value_dim % 4 == 0 and dim <= self._ops.distie_decay_scan_chunked_max_dim():
+            # portions of prompts: chunks of rows side by side instead of one row after the other. Which rows form
+            # a chunk is worked out here from the step's row counts (known on the host outside captured steps).
+            key = ("scan_chunks", num_heads, dim, value_dim)
+            plan = meta.scratch.get(key)
+            if plan is None:
+                rows = self._ops.distie_decay_scan_chunk_rows()
+                cu = np.asarray(meta.host_cu_q, dtype=np.int64)
+                table, first = [], [0]
+                for b in range(meta.num_requests):
+                    for at in range(int(cu[b]), int(cu[b + 1]), rows):
+                        table.append((b, at, min(rows, int(cu[b + 1]) - at), 0))
+                    first.append(len(table))
+                packed = self.upload(np.concatenate([np.asarray(table, dtype=np.int32).reshape(-1),
+                                                     np.asarray(first, dtype=np.int32)]))
+                scratch = torch.empty((len(table), num_heads, dim, value_dim), dtype=torch.float32, device=self.device)
+                plan = meta.scratch[key] = (len(table), packed, scratch)
+            count, packed, scratch = plan
+            _check(self._ops.distie_decay_scan_chunked(
+                product.data_ptr(), _code(product), W, state.data_ptr(), decay.data_ptr(), out.data_ptr(),
+                scratch.data_ptr(), packed.data_ptr(), packed.data_ptr() + 16 * count, meta.state_slots.data_ptr(),
+                count, meta.num_requests, num_heads, dim, value_dim, self._stream()), "decay_scan_chunked")
+            _mark_written(state)
+            return out
         _check(self._ops.distie_decay_scan(product.data_ptr(), _code(product), W, state.data_ptr(), decay.data_ptr(),
                                            out.data_ptr(), meta.cu_q.data_ptr(), meta.state_slots.data_ptr(),
                                            meta.num_requests, num_heads, dim, value_dim, self._stream()), "decay_scan")
@@ -1175,11 +1215,15 @@ class HipOps(Ops):
     def activation(self, x, kind):
         if kind not in self.ACTIVATIONS:
             raise KernelError(f"no activation named {kind!r}")
-        x = self.dense(x)
-        self._own(x)
-        out = torch.empty_like(x)
-        _check(self._ops.distie_activation(x.data_ptr(), out.data_ptr(), _code(x), x.numel(), self.ACTIVATIONS[kind],
-                                           self._stream()), "activation")
+        if isinstance(x, (PendingNorm, PendingProduct)):
+            x = self.dense(x)
+        slices, source, dtype = 1, x, x.dtype
+        if isinstance(x, PartialSums):
+            slices, source = x.slices, x.data
+        self._own(source)
+        out = torch.empty(tuple(x.shape), dtype=dtype, device=self.device)
+        _check(self._ops.distie_activation(source.data_ptr(), _code(source), slices, out.data_ptr(), _code(out), out.numel(),
+                                           self.ACTIVATIONS[kind], self._stream()), "activation")
         return out
 
     def silu_mul(self, gate_up):

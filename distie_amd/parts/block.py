@@ -142,7 +142,7 @@ class HyperConnections(Block):
     def forward(self, ops, stream: ResidualStream, ctx: StepContext, cache, writes_cache: bool) -> None:
         self._constants(stream.hidden.device)
         h = self._enter(ops, stream, 1, self.mixer_norm, ctx.act_dtype)
-        gate = ops.dense(ops.linear(h, self.gate_weight[1], self.gate_bias[1])) if self.gated else None
+        gate = ops.linear(h, self.gate_weight[1], self.gate_bias[1]) if self.gated else None
         if self.input_taps:
             history = cache["input_conv"]["history"] if self.input_taps > 1 else None
             h = ops.causal_conv(h, self.input_filter, history, ctx.meta, residual=True)
@@ -151,7 +151,7 @@ class HyperConnections(Block):
         if self.feed_forward is None:
             return
         h = self._enter(ops, stream, 2, self.feed_forward_norm, ctx.act_dtype)
-        gate = ops.dense(ops.linear(h, self.gate_weight[2], self.gate_bias[2])) if self.gated else None
+        gate = ops.linear(h, self.gate_weight[2], self.gate_bias[2]) if self.gated else None
         y = self.feed_forward.forward(ops, h, ctx)
         stream.lanes["pending"] = (y, gate, self.mix[2], self.write[2])
 

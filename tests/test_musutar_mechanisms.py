@@ -137,19 +137,26 @@ def test_convolution_over_time_with_carried_inputs(ops, taps, residual):
             close(got, gather(want, rows), dtype, f"taps {taps} rows {rows}")
 
 
-@pytest.mark.parametrize("heads,dim,vdim", [(2, 8, 16), (3, 16, 8), (1, 32, 32), (2, 40, 72)])
-def test_decayed_state_scan(ops, heads, dim, vdim):
+LONG_LENGTHS = (150, 1, 70, 33)
+LONG_CUTS = ((100, 1, 2, 0), (17, 0, 64, 33), (33, 0, 4, 0))
+
+
+@pytest.mark.parametrize("lengths,cuts", [(LENGTHS, CUTS), (LONG_LENGTHS, LONG_CUTS)])
+@pytest.mark.parametrize("heads,dim,vdim", [(2, 8, 16), (3, 16, 8), (1, 32, 32), (2, 40, 72), (2, 128, 64)])
+def test_decayed_state_scan(ops, heads, dim, vdim, lengths, cuts):
+    """Short portions go row after row, long ones in chunks of rows worked side by side (on the GPU): the same
+    recurrence either way, with the state handed from step to step."""
     decay = torch.tensor([0.999, 0.6, 0.9][:heads], dtype=torch.float32)
     width = heads * (2 * dim + vdim) + 5                       # further columns are left alone
     for dtype in act_types(ops):
-        seqs = [rnd(n, width, seed=20 + i).to(dtype) for i, n in enumerate(LENGTHS)]
+        seqs = [rnd(n, width, seed=20 + i).to(dtype) for i, n in enumerate(lengths)]
         want = []
         for s in seqs:
             z = plain.silu(s.to(F))
             q, k = z[:, :heads * dim].view(-1, heads, dim), z[:, heads * dim:2 * heads * dim].view(-1, heads, dim)
             v = z[:, 2 * heads * dim:heads * (2 * dim + vdim)].view(-1, heads, vdim)
             want.append(plain.decayed_state_scan(q, k, v, decay.tolist()).reshape(-1, heads * vdim))
-        steps = Steps(ops, FixedState.of((heads, dim, vdim)), LENGTHS, CUTS)
+        steps = Steps(ops, FixedState.of((heads, dim, vdim)), lengths, cuts)
         for meta, rows in steps:
             got = ops.decay_scan(gather(seqs, rows).to(ops.device), steps.view()["state"], decay.to(ops.device), meta,
                                  heads, dim, vdim)
