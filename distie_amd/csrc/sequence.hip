@@ -16,6 +16,11 @@ constexpr int MAX_TAPS = 16;
 
 __device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + __expf(-x)); }
 __device__ __forceinline__ float siluf(float x) { return x / (1.f + __expf(-x)); }
+// two values rounded to bfloat16 as one 32-bit word (the first in the low half)
+__device__ __forceinline__ uint32_t bf16_word(float lo, float hi) {
+  return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(lo))) |
+         (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(hi))) << 16);
+}
 
 // ---------------------------------------------------------------------------------------------------
 // Residual streams. streams float32 [T, S, C]. In this order, each step optional:
@@ -24,7 +29,54 @@ __device__ __forceinline__ float siluf(float x) { return x / (1.f + __expf(-x));
 //   read:   u = sum_s in_w[s] x_s;  h = norm(u) * weight                (kind 0: u itself, 1: centred, 2: root mean square)
 // One block a token; u of the whole row waits in LDS between the two passes of the statistics.
 // MS: the most streams this instance takes (its loops are unrolled to that, so the streams stay in registers).
-template <int MS, typename Y, typename G, typename W, typename H>
+// V: channels a thread takes at a time, 4 (16-byte loads of float32, 8-byte loads of bfloat16; the width must be a
+// multiple of 4) or 1. With V = 4 a row of up to 4 x the block's threads is loaded in one go, every load under way
+// at once, which is what a step of few rows waits for.
+template <int V, typename T>
+__device__ __forceinline__ void loadv(const T* __restrict__ p, float out[V]) {
+  if constexpr (V == 4 && sizeof(T) == 4) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    out[0] = v.x, out[1] = v.y, out[2] = v.z, out[3] = v.w;
+  } else if constexpr (V == 4) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    out[0] = __uint_as_float(v.x << 16), out[1] = __uint_as_float(v.x & 0xffff0000u);
+    out[2] = __uint_as_float(v.y << 16), out[3] = __uint_as_float(v.y & 0xffff0000u);
+  } else {
+#pragma unroll
+    for (int k = 0; k < V; ++k) out[k] = to_float(p[k]);
+  }
+}
+
+template <int V, typename T>
+__device__ __forceinline__ void storev(T* __restrict__ p, const float v[V]) {
+  if constexpr (V == 4 && sizeof(T) == 4) {
+    *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
+  } else if constexpr (V == 4) {
+    *reinterpret_cast<uint2*>(p) = uint2{bf16_word(v[0], v[1]), bf16_word(v[2], v[3])};
+  } else {
+#pragma unroll
+    for (int k = 0; k < V; ++k) p[k] = from_float<T>(v[k]);
+  }
+}
+
+// the sum of `slices` vectors that lie `stride` elements apart, added in order
+template <int V, typename T>
+__device__ __forceinline__ void sumv(const T* __restrict__ p, int slices, int64_t stride, float out[V]) {
+  loadv<V>(p, out);
+  for (int s = 1; s < slices; s += 4) {
+    float a[4][V];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) loadv<V>(p + min(s + u, slices - 1) * stride, a[u]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (s + u < slices) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) out[k] += a[u][k];
+      }
+  }
+}
+
+template <int MS, int V, typename Y, typename G, typename W, typename H>
 __global__ void hyper_step_kernel(float* __restrict__ streams, int S, const float* __restrict__ init, const Y* __restrict__ y,
                                   int y_slices, int64_t y_slice_stride, const G* __restrict__ gate, int64_t gate_ld,
                                   int gate_slices, int64_t gate_slice_stride,
@@ -44,47 +96,61 @@ __global__ void hyper_step_kernel(float* __restrict__ streams, int S, const floa
     for (int j = 0; j < MS; ++j) m[i][j] = (y != nullptr && i < S && j < S) ? mix[i * S + j] : 0.f;
   }
   float sum = 0.f;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float v[MS];
-    if (init != nullptr) {
-      const float e = init[t * C + c];
+  for (int c = V * threadIdx.x; c < C; c += V * blockDim.x) {
+    float v[MS][V];
 #pragma unroll
-      for (int s = 0; s < MS; ++s) v[s] = s < S ? e : 0.f;
-    } else {
+    for (int s = 0; s < MS; ++s) {
+      if (s < S) {
+        loadv<V>(init != nullptr ? init + t * C + c : x + s * C + c, v[s]);
+      } else {
 #pragma unroll
-      for (int s = 0; s < MS; ++s) v[s] = s < S ? x[s * C + c] : 0.f;
+        for (int k = 0; k < V; ++k) v[s][k] = 0.f;
+      }
     }
     if (y != nullptr) {
-      float d = sum_strided(y + t * C + c, y_slices, y_slice_stride);
-      if (gate != nullptr) d *= sigmoidf(sum_strided(gate + t * gate_ld + c, gate_slices, gate_slice_stride));
-      float n[MS];
+      float d[V];
+      sumv<V>(y + t * C + c, y_slices, y_slice_stride, d);
+      if (gate != nullptr) {
+        float g[V];
+        sumv<V>(gate + t * gate_ld + c, gate_slices, gate_slice_stride, g);
 #pragma unroll
-      for (int j = 0; j < MS; ++j) {
-        float a = 0.f;
-#pragma unroll
-        for (int s = 0; s < MS; ++s) a += m[s][j] * v[s];
-        n[j] = a + ow[j] * d;
+        for (int k = 0; k < V; ++k) d[k] *= sigmoidf(g[k]);
       }
+      float n[MS][V];
 #pragma unroll
-      for (int j = 0; j < MS; ++j) v[j] = n[j];
+      for (int j = 0; j < MS; ++j)
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+          float a = 0.f;
+#pragma unroll
+          for (int s = 0; s < MS; ++s) a += m[s][j] * v[s][k];
+          n[j][k] = a + ow[j] * d[k];
+        }
+#pragma unroll
+      for (int j = 0; j < MS; ++j)
+#pragma unroll
+        for (int k = 0; k < V; ++k) v[j][k] = n[j][k];
     }
     if (init != nullptr || y != nullptr) {
 #pragma unroll
       for (int s = 0; s < MS; ++s)
-        if (s < S) x[s * C + c] = v[s];
+        if (s < S) storev<V>(x + s * C + c, v[s]);
     }
     if (h != nullptr) {
-      float u = 0.f;
 #pragma unroll
-      for (int s = 0; s < MS; ++s) u += iw[s] * v[s];
-      row[c] = u;
-      sum += kind == 2 ? u * u : u;
+      for (int k = 0; k < V; ++k) {
+        float u = 0.f;
+#pragma unroll
+        for (int s = 0; s < MS; ++s) u += iw[s] * v[s][k];
+        row[c + k] = u;
+        sum += kind == 2 ? u * u : u;
+      }
     }
   }
   if (h == nullptr) return;
   H* out = h + t * C;
   if (kind == 0) {
-    for (int c = threadIdx.x; c < C; c += blockDim.x) out[c] = from_float<H>(row[c]);
+    for (int c = V * threadIdx.x; c < C; c += V * blockDim.x) storev<V>(out + c, row + c);
     return;
   }
   sum = block_sum(sum, scratch);
@@ -92,17 +158,25 @@ __global__ void hyper_step_kernel(float* __restrict__ streams, int S, const floa
   if (kind == 1) {
     mean = sum / C;
     float dev = 0.f;
-    for (int c = threadIdx.x; c < C; c += blockDim.x) {
-      const float d = row[c] - mean;
-      dev += d * d;
+    for (int c = V * threadIdx.x; c < C; c += V * blockDim.x) {
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        const float d = row[c + k] - mean;
+        dev += d * d;
+      }
     }
     dev = block_sum(dev, scratch);
     scale = 1.f / sqrtf(dev / C + eps);
   } else {
     scale = 1.f / sqrtf(sum / C + eps);
   }
-  for (int c = threadIdx.x; c < C; c += blockDim.x)
-    out[c] = from_float<H>((row[c] - mean) * scale * to_float(norm_w[c]));
+  for (int c = V * threadIdx.x; c < C; c += V * blockDim.x) {
+    float w[V], r[V];
+    loadv<V>(norm_w + c, w);
+#pragma unroll
+    for (int k = 0; k < V; ++k) r[k] = (row[c + k] - mean) * scale * w[k];
+    storev<V>(out + c, r);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -365,6 +439,263 @@ decay_scan_kernel(const X* __restrict__ product, int64_t ld, float* __restrict__
 }
 
 // ---------------------------------------------------------------------------------------------------
+// bfloat16 with 16-byte loads and stores: eight channels a thread. Values are put together as whole 32-bit words.
+__device__ __forceinline__ void unpack_bf16x8(const uint4& raw, float v[8]) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    v[2 * e] = __uint_as_float(w[e] << 16);
+    v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ uint32_t bf16_bits(float x) {
+  return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(x)));
+}
+__device__ __forceinline__ uint4 pack_bf16x8(const float v[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) w[e] = bf16_bits(v[2 * e]) | (bf16_bits(v[2 * e + 1]) << 16);
+  return uint4{w[0], w[1], w[2], w[3]};
+}
+__device__ __forceinline__ uint4 load16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+
+// the convolution at eight channels c0 .. c0 + 7 of row t (filters of `taps` taps, bfloat16, [N, taps])
+__device__ __forceinline__ void conv8(const bf16_t* __restrict__ x, int64_t ldx, const float* __restrict__ state,
+                                      const bf16_t* __restrict__ weight, int taps, int64_t t, int i, int c0, int N,
+                                      float acc[8], float self[8]) {
+  unpack_bf16x8(load16(x + t * ldx + c0), self);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  if (taps < 1) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = self[e];
+    return;
+  }
+  for (int j = 0; j < taps; ++j) {
+    const int back = taps - 1 - j;
+    float v[8];
+    if (back == 0) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = self[e];
+    } else if (back <= i) {
+      unpack_bf16x8(load16(x + (t - back) * ldx + c0), v);
+    } else {
+      const float4* p = reinterpret_cast<const float4*>(state + static_cast<int64_t>(taps - 1 - (back - i)) * N + c0);
+      const float4 lo = p[0], hi = p[1];
+      v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += to_float(weight[static_cast<int64_t>(c0 + e) * taps + j]) * v[e];
+  }
+}
+
+// a request that brings one row: its state of eight channels moved on by that row
+__device__ __forceinline__ void shift_state8(float* __restrict__ own, int taps, int c0, int N, const float self[8]) {
+  float4 keep[MAX_TAPS][2];
+  for (int k = 1; k < taps - 1; ++k) {
+    const float4* p = reinterpret_cast<const float4*>(own + static_cast<int64_t>(k) * N + c0);
+    keep[k][0] = p[0], keep[k][1] = p[1];
+  }
+  for (int k = 1; k < taps - 1; ++k) {
+    float4* p = reinterpret_cast<float4*>(own + static_cast<int64_t>(k - 1) * N + c0);
+    p[0] = keep[k][0], p[1] = keep[k][1];
+  }
+  float4* last = reinterpret_cast<float4*>(own + static_cast<int64_t>(taps - 2) * N + c0);
+  last[0] = float4{self[0], self[1], self[2], self[3]};
+  last[1] = float4{self[4], self[5], self[6], self[7]};
+}
+
+__global__ void causal_conv_bf16x8_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ weight,
+                                          int taps, float* __restrict__ state, bf16_t* __restrict__ out, int64_t ldo,
+                                          int residual, const int32_t* __restrict__ cu_q,
+                                          const int32_t* __restrict__ token_request,
+                                          const int32_t* __restrict__ state_slots, int N) {
+  const int64_t t = blockIdx.x;
+  const int c0 = 8 * (blockIdx.y * blockDim.x + threadIdx.x);
+  if (c0 >= N) return;
+  const int b = token_request[t];
+  const int first = cu_q[b];
+  const int i = static_cast<int>(t) - first;
+  float* own = state + static_cast<int64_t>(state_slots[b]) * (taps - 1) * N;
+  float acc[8], self[8];
+  conv8(x, ldx, own, weight, taps, t, i, c0, N, acc, self);
+  if (residual) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += self[e];
+  }
+  *reinterpret_cast<uint4*>(out + t * ldo + c0) = pack_bf16x8(acc);
+  if (cu_q[b + 1] - first == 1 && taps > 1) shift_state8(own, taps, c0, N, self);
+}
+
+// conv_rope_kv_write for bfloat16 products and caches, D, E and the number of pairs multiples of 8, DP == D or the
+// places beyond D zeroed by eight. Blocks 0 .. T-1: q and k of one token (a thread turns eight pairs, or copies eight
+// single dimensions). The blocks behind them: v for 16 tokens each; a thread owns one channel of v and, where
+// the 16 tokens lie side by side in one page, writes their values as one run of 32 bytes (the cache keeps v with
+// the key index innermost).
+constexpr int VGROUP = 16;
+
+__global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ product, int64_t ld, const bf16_t* __restrict__ weight,
+                                               int taps, float* __restrict__ state, const float2* __restrict__ table,
+                                               int pairs, float magnitude, bf16_t* __restrict__ q_out,
+                                               bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
+                                               const int32_t* __restrict__ slots, const int32_t* __restrict__ cu_q,
+                                               const int32_t* __restrict__ token_request,
+                                               const int32_t* __restrict__ state_slots, int T, int H, int G, int D, int E,
+                                               int DP, int block_size, int has_kv, int write) {
+  const int N = H * D + (has_kv ? G * (D + E) : 0);
+  if (static_cast<int>(blockIdx.x) >= T) {
+    // ---- v: 16 tokens, one channel a thread
+    const int t0 = (static_cast<int>(blockIdx.x) - T) * VGROUP;
+    const int n = min(VGROUP, T - t0);
+    const int64_t slot0 = write ? slots[t0] : 0;
+    bool together = write && n == VGROUP && block_size % 8 == 0 && slot0 % block_size % 8 == 0 &&
+                    slot0 % block_size + VGROUP <= block_size;
+    if (write) {
+#pragma unroll
+      for (int k = 1; k < VGROUP; ++k) together = together && slots[min(t0 + k, T - 1)] == slot0 + k;
+    }
+    uint16_t* cache = reinterpret_cast<uint16_t*>(v_cache);
+    for (int item = threadIdx.x; item < G * E; item += blockDim.x) {
+      const int g = item / E, e = item % E;
+      const int c = (H + G) * D + item;
+      float w[MAX_TAPS];
+      for (int j = 0; j < taps; ++j) w[j] = to_float(weight[static_cast<int64_t>(c) * taps + j]);
+      uint32_t bits[VGROUP];
+#pragma unroll
+      for (int k = 0; k < VGROUP; ++k) {
+        bits[k] = 0;
+        if (k >= n) continue;
+        const int64_t t = t0 + k;
+        const int b = token_request[t];
+        const int first = cu_q[b];
+        const int i = static_cast<int>(t) - first;
+        float* own = taps > 1 ? state + static_cast<int64_t>(state_slots[b]) * (taps - 1) * N : nullptr;
+        const float self = to_float(product[t * ld + c]);
+        const float v = taps < 1 ? self : conv_at(product, ld, own, w, taps, t, i, c, N);
+        bits[k] = bf16_bits(v);
+        if (taps > 1 && cu_q[b + 1] - first == 1) {
+          float keep[MAX_TAPS];
+          for (int m = 1; m < taps - 1; ++m) keep[m] = own[static_cast<int64_t>(m) * N + c];
+          for (int m = 1; m < taps - 1; ++m) own[static_cast<int64_t>(m - 1) * N + c] = keep[m];
+          own[static_cast<int64_t>(taps - 2) * N + c] = self;
+        }
+      }
+      if (!write) continue;
+      if (together) {
+        const int64_t page = slot0 / block_size;
+        uint16_t* dst = cache + ((page * G + g) * DP + e) * block_size + slot0 % block_size;
+        *reinterpret_cast<uint4*>(dst) = uint4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16),
+                                               bits[4] | (bits[5] << 16), bits[6] | (bits[7] << 16)};
+        *reinterpret_cast<uint4*>(dst + 8) = uint4{bits[8] | (bits[9] << 16), bits[10] | (bits[11] << 16),
+                                                   bits[12] | (bits[13] << 16), bits[14] | (bits[15] << 16)};
+      } else {
+#pragma unroll
+        for (int k = 0; k < VGROUP; ++k) {
+          if (k >= n) break;
+          const int64_t slot = slots[t0 + k];
+          cache[((slot / block_size * G + g) * DP + e) * block_size + slot % block_size] = static_cast<uint16_t>(bits[k]);
+        }
+      }
+    }
+    return;
+  }
+  // ---- q and k of token t
+  const int64_t t = blockIdx.x;
+  const int b = token_request[t];
+  const int first = cu_q[b];
+  const int i = static_cast<int>(t) - first;
+  const bool single = cu_q[b + 1] - first == 1 && taps > 1;
+  float* own = taps > 1 ? state + static_cast<int64_t>(state_slots[b]) * (taps - 1) * N : nullptr;
+  const int64_t slot = (has_kv && write) ? slots[t] : 0;
+  const int64_t page = slot / block_size;
+  const int offset = static_cast<int>(slot % block_size);
+  const int turned = has_kv ? H + G : H;
+  const int pair8 = pairs / 8, rest8 = (DP - 2 * pairs) / 8;
+  const int per_head = pair8 + rest8;
+  for (int item = threadIdx.x; item < turned * per_head; item += blockDim.x) {
+    const int head = item / per_head;
+    const int j8 = item % per_head;
+    const int base = head * D;
+    bf16_t* dst = head < H ? q_out + (t * H + head) * DP
+                           : k_cache + ((page * G + (head - H)) * block_size + offset) * DP;
+    const bool store = head < H || write;
+    if (j8 < pair8) {
+      const int d0 = 8 * j8, d1 = d0 + pairs;
+      float x0[8], x1[8], s0[8], s1[8], a[8], c[8];
+      conv8(product, ld, own, weight, taps, t, i, base + d0, N, x0, s0);
+      conv8(product, ld, own, weight, taps, t, i, base + d1, N, x1, s1);
+      const float4* angles = reinterpret_cast<const float4*>(table + t * pairs + d0);       // (cos, sin) x 8
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float4 cs = angles[e];
+        a[2 * e] = x0[2 * e] * (cs.x * magnitude) - x1[2 * e] * (cs.y * magnitude);
+        c[2 * e] = x1[2 * e] * (cs.x * magnitude) + x0[2 * e] * (cs.y * magnitude);
+        a[2 * e + 1] = x0[2 * e + 1] * (cs.z * magnitude) - x1[2 * e + 1] * (cs.w * magnitude);
+        c[2 * e + 1] = x1[2 * e + 1] * (cs.z * magnitude) + x0[2 * e + 1] * (cs.w * magnitude);
+      }
+      if (store) {
+        *reinterpret_cast<uint4*>(dst + d0) = pack_bf16x8(a);
+        *reinterpret_cast<uint4*>(dst + d1) = pack_bf16x8(c);
+      }
+      if (single) {
+        shift_state8(own, taps, base + d0, N, s0);
+        shift_state8(own, taps, base + d1, N, s1);
+      }
+    } else {
+      const int d0 = 2 * pairs + 8 * (j8 - pair8);
+      float a[8] = {}, s0[8];
+      if (d0 < D) {
+        conv8(product, ld, own, weight, taps, t, i, base + d0, N, a, s0);
+        if (single) shift_state8(own, taps, base + d0, N, s0);
+      }
+      if (head < H || (write && d0 < D)) *reinterpret_cast<uint4*>(dst + d0) = pack_bf16x8(a);
+    }
+  }
+}
+
+// out = x * sigmoid(gates), eight a thread
+__global__ void sigmoid_gate_bf16x8_kernel(const bf16_t* __restrict__ x, int ldh, int E, const bf16_t* __restrict__ gates,
+                                           int64_t ldg, bf16_t* __restrict__ out, int width, int64_t T) {
+  const int width8 = width / 8;
+  const int64_t total = T * width8;
+  for (int64_t it = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; it < total;
+       it += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t t = it / width8;
+    const int c = 8 * static_cast<int>(it % width8);
+    const int head = c / E, e = c % E;
+    float v[8], g[8];
+    unpack_bf16x8(load16(x + (t * (width / E) + head) * ldh + e), v);
+    unpack_bf16x8(load16(gates + t * ldg + c), g);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] *= sigmoidf(g[k]);
+    *reinterpret_cast<uint4*>(out + t * width + c) = pack_bf16x8(v);
+  }
+}
+
+__global__ void activation_bf16x8_kernel(const uint4* __restrict__ in, uint4* __restrict__ out, int64_t count8, int kind) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < count8;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    float v[8];
+    unpack_bf16x8(in[i], v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float z = v[k];
+      if (kind == 0) {
+        const float p = fmaxf(z, 0.f);
+        v[k] = p * p;
+      } else if (kind == 1) {
+        v[k] = siluf(z);
+      } else if (kind == 2) {
+        v[k] = 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+      } else {
+        v[k] = fmaxf(z, 0.f);
+      }
+    }
+    out[i] = pack_bf16x8(v);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
 // The same recurrence over portions of prompts, in chunks of 64 rows that run side by side. With L the rows of a
 // chunk, S the state in front of it and w^m the decay's powers (a table made by repeated multiplication):
 //   sums:     P[d][e]   = sum_j w^(L-1-j) k_j[d] v_j[e]                      (each chunk alone)
@@ -580,7 +911,13 @@ extern "C" int distie_hyper_step(float* streams, int S, const float* init, const
   if (S < 1 || S > MAX_STREAMS || C < 1 || kind < 0 || kind > 2 || y_slices < 1 || gate_slices < 1) return DISTIE_BAD_ARGUMENT;
   if (y != nullptr && (mix == nullptr || out_w == nullptr)) return DISTIE_BAD_ARGUMENT;
   if (h != nullptr && (in_w == nullptr || (kind != 0 && norm_w == nullptr))) return DISTIE_BAD_ARGUMENT;
-  const int threads = C >= 2048 ? 512 : (C >= 512 ? 256 : (C >= 128 ? 128 : 64));
+  // 16-byte pieces where every row of every operand starts at a multiple of 16 bytes
+  const bool wide = C % 8 == 0 && gate_ld % 8 == 0 && reinterpret_cast<uintptr_t>(streams) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(init) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(gate) % 16 == 0 && reinterpret_cast<uintptr_t>(norm_w) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(h) % 16 == 0;
+  const int per = wide ? C / 4 : C;
+  const int threads = per >= 1024 ? 1024 : (per >= 512 ? 512 : (per >= 256 ? 256 : (per >= 128 ? 128 : 64)));
   const size_t lds = h != nullptr ? static_cast<size_t>(C) * sizeof(float) : 0;
   const int64_t y_stride = static_cast<int64_t>(T) * C;
   if (y == nullptr) y_dtype = DISTIE_F32;
@@ -588,11 +925,17 @@ extern "C" int distie_hyper_step(float* streams, int S, const float* init, const
   if (norm_w == nullptr) norm_dtype = DISTIE_F32;
   if (h == nullptr) h_dtype = DISTIE_F32;
   if (lds > 48 * 1024) return DISTIE_BAD_ARGUMENT;      // a row of u waits in LDS: widths up to 12,288
-#define DISTIE_HYPER(MS)                                                                                               \
+#define DISTIE_HYPER_V(MS, V)                                                                                          \
   DISTIE_DISPATCH(y_dtype, Y, DISTIE_DISPATCH(gate_dtype, G, DISTIE_DISPATCH(norm_dtype, W, DISTIE_DISPATCH(h_dtype, HT,  \
-      hyper_step_kernel<MS, Y, G, W, HT><<<T, threads, lds, stream>>>(                                                \
+      hyper_step_kernel<MS, V, Y, G, W, HT><<<T, threads, lds, stream>>>(                                             \
           streams, S, init, static_cast<const Y*>(y), y_slices, y_stride, static_cast<const G*>(gate), gate_ld,       \
           gate_slices, gate_ld * T, mix, out_w, in_w, static_cast<const W*>(norm_w), kind, eps, static_cast<HT*>(h), C)))))
+#define DISTIE_HYPER(MS)   \
+  if (wide) {              \
+    DISTIE_HYPER_V(MS, 4); \
+  } else {                 \
+    DISTIE_HYPER_V(MS, 1); \
+  }
   if (S == 1) {
     DISTIE_HYPER(1);
   } else if (S == 2) {
@@ -602,6 +945,7 @@ extern "C" int distie_hyper_step(float* streams, int S, const float* init, const
   } else {
     DISTIE_HYPER(8);
   }
+#undef DISTIE_HYPER_V
 #undef DISTIE_HYPER
   return launch_status();
 }
@@ -612,6 +956,15 @@ extern "C" int distie_causal_conv(const void* x, int x_dtype, int64_t ldx, const
                                   hipStream_t stream) {
   if (T <= 0) return 0;
   if (taps < 1 || taps > MAX_TAPS || N < 1 || ldx < N || ldo < N || (taps > 1 && state == nullptr)) return DISTIE_BAD_ARGUMENT;
+  if (x_dtype == DISTIE_BF16 && w_dtype == DISTIE_BF16 && out_dtype == DISTIE_BF16 && N % 8 == 0 && ldx % 8 == 0 &&
+      ldo % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && reinterpret_cast<uintptr_t>(state) % 16 == 0) {
+    const int items = N / 8;
+    const int threads8 = items >= 256 ? 256 : (items >= 128 ? 128 : 64);
+    causal_conv_bf16x8_kernel<<<dim3(T, (items + threads8 - 1) / threads8), threads8, 0, stream>>>(
+        static_cast<const bf16_t*>(x), ldx, static_cast<const bf16_t*>(weight), taps, state, static_cast<bf16_t*>(out), ldo,
+        residual, cu_q, token_request, state_slots, N);
+    return launch_status();
+  }
   const int threads = N >= 256 ? 256 : (N >= 128 ? 128 : 64);
   const dim3 grid(T, (N + threads - 1) / threads);
   DISTIE_DISPATCH(x_dtype, X, DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(out_dtype, O,
@@ -645,6 +998,18 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
   if ((pairs > 0 && table == nullptr) || (taps > 1 && state == nullptr) || (taps >= 1 && weight == nullptr))
     return DISTIE_BAD_ARGUMENT;
   if (has_kv && write && (k_cache == nullptr || v_cache == nullptr || slots == nullptr)) return DISTIE_BAD_ARGUMENT;
+  if (dtype == DISTIE_BF16 && (weight == nullptr || w_dtype == DISTIE_BF16) && (!write || cache_dtype == DISTIE_BF16) &&
+      D % 8 == 0 && E % 8 == 0 && DP % 8 == 0 && pairs % 8 == 0 && ld % 8 == 0 &&
+      reinterpret_cast<uintptr_t>(product) % 16 == 0 && reinterpret_cast<uintptr_t>(q_out) % 16 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(state) % 16 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0) {
+    const int items = (has_kv ? H + G : H) * ((DP - pairs) / 8);
+    const int threads8 = items > 128 ? 256 : (items > 64 ? 128 : 64);
+    const int v_blocks = has_kv && (write || taps > 1) ? (T + VGROUP - 1) / VGROUP : 0;
+    conv_rope_kv_write_bf16_kernel<<<T + v_blocks, threads8, 0, stream>>>(
+        static_cast<const bf16_t*>(product), ld, static_cast<const bf16_t*>(weight), taps, state,
+        static_cast<const float2*>(table), pairs, magnitude, static_cast<bf16_t*>(q_out), static_cast<bf16_t*>(k_cache),
+        static_cast<bf16_t*>(v_cache), slots, cu_q, token_request, state_slots, T, H, G, D, E, DP, block_size, has_kv, write);
+    return launch_status();
+  }
   const int work = DP - pairs > E ? DP - pairs : E;
   const int threads = work > 128 ? 256 : (work > 64 ? 128 : 64);
   const dim3 grid(T, has_kv ? H + 2 * G : H);
@@ -661,6 +1026,15 @@ extern "C" int distie_sigmoid_gate(const void* x, int x_dtype, int ldh, int E, c
                                    void* out, int out_dtype, int T, int width, hipStream_t stream) {
   if (T <= 0) return 0;
   if (E < 1 || width < 1 || width % E || ldh < E || ldg < width) return DISTIE_BAD_ARGUMENT;
+  if (x_dtype == DISTIE_BF16 && g_dtype == DISTIE_BF16 && out_dtype == DISTIE_BF16 && E % 8 == 0 && ldh % 8 == 0 &&
+      ldg % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(gates) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+    const int64_t pieces = static_cast<int64_t>(T) * (width / 8);
+    const int blocks8 = static_cast<int>(pieces / 256 + 1 < 16384 ? pieces / 256 + 1 : 16384);
+    sigmoid_gate_bf16x8_kernel<<<blocks8, 256, 0, stream>>>(static_cast<const bf16_t*>(x), ldh, E,
+                                                            static_cast<const bf16_t*>(gates), ldg,
+                                                            static_cast<bf16_t*>(out), width, T);
+    return launch_status();
+  }
   const int threads = width >= 256 ? 256 : (width >= 128 ? 128 : 64);
   const dim3 grid(T, (width + threads - 1) / threads);
   DISTIE_DISPATCH(x_dtype, X, DISTIE_DISPATCH(g_dtype, G, DISTIE_DISPATCH(out_dtype, O,
@@ -685,6 +1059,12 @@ extern "C" int distie_activation(const void* in, int in_dtype, int slices, void*
                                  hipStream_t stream) {
   if (count <= 0) return 0;
   if (kind < 0 || kind > 3 || slices < 1) return DISTIE_BAD_ARGUMENT;
+  if (in_dtype == DISTIE_BF16 && dtype == DISTIE_BF16 && slices == 1 && count % 8 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+    const int64_t pieces = count / 8;
+    const int blocks8 = static_cast<int>(pieces / 256 + 1 < 16384 ? pieces / 256 + 1 : 16384);
+    activation_bf16x8_kernel<<<blocks8, 256, 0, stream>>>(static_cast<const uint4*>(in), static_cast<uint4*>(out), pieces, kind);
+    return launch_status();
+  }
   const int threads = 256;
   const int64_t blocks = (count + threads - 1) / threads;
   if (blocks > 0x7fffffff) return DISTIE_BAD_ARGUMENT;

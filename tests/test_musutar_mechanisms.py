@@ -182,10 +182,11 @@ def test_gates_norm_and_activations(ops):
             close(ops.activation(z.to(ops.device), kind), f(z.to(F)), dtype, kind)
 
 
-@pytest.mark.parametrize("heads,kv_heads,dim,vdim,rot,taps,window,lends", [
-    (4, 2, 16, 24, 8, 4, 6, True), (2, 2, 32, 32, 32, 1, None, False), (3, 1, 40, 16, 0, 3, 9, False),
-    (2, 1, 16, 16, 16, 0, 4, True)])
-def test_attention_mixer(ops, heads, kv_heads, dim, vdim, rot, taps, window, lends):
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim,rot,taps,window,lends,lengths,cuts", [
+    (4, 2, 16, 24, 8, 4, 6, True, LENGTHS, CUTS), (2, 2, 32, 32, 32, 1, None, False, LENGTHS, CUTS),
+    (3, 1, 40, 16, 0, 3, 9, False, LENGTHS, CUTS), (2, 1, 16, 16, 16, 0, 4, True, LENGTHS, CUTS),
+    (4, 2, 64, 64, 32, 4, 40, True, LONG_LENGTHS, LONG_CUTS), (2, 1, 64, 32, 64, 3, 21, False, LONG_LENGTHS, LONG_CUTS)])
+def test_attention_mixer(ops, heads, kv_heads, dim, vdim, rot, taps, window, lends, lengths, cuts):
     """The mixer alone over a batch in steps: projections, convolutions with carried inputs, partial rotation with
     scaled frequencies, the cache write, the window, the output gate; and a second mixer that borrows the first one's
     keys and values with a longer window of its own."""
@@ -208,9 +209,9 @@ def test_attention_mixer(ops, heads, kv_heads, dim, vdim, rot, taps, window, len
             part.load({k: v.to(ops.device) for k, v in w.items()})
             weights.append({"m." + k: v for k, v in w.items()})
         assert "k" not in weights[-1] or not lends
-        cache = CacheManager([{"mixer": p.cache_requirement()} for p in parts], 4, 64, 5, device=ops.device, dtype=dtype)
+        cache = CacheManager([{"mixer": p.cache_requirement()} for p in parts], 16, 64, 5, device=ops.device, dtype=dtype)
         builder = BatchBuilder(cache, 512, ops.device, 1000)
-        seqs = [rnd(n, C, seed=50 + i).to(dtype) for i, n in enumerate(LENGTHS)]
+        seqs = [rnd(n, C, seed=50 + i).to(dtype) for i, n in enumerate(lengths)]
         cfg = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": 0.2, "rot": rot_cfg,
                "mask": {"size": window} if window else None}
         want = [[], []]
@@ -222,14 +223,14 @@ def test_attention_mixer(ops, heads, kv_heads, dim, vdim, rot, taps, window, len
                 theirs = {**cfg, "heads": heads * 2, "mask": {"size": longer} if longer else None}
                 want[1].append(plain.attention_mixer(s.to(F), {k: v.to(F) for k, v in weights[1].items()}, "m.",
                                                      theirs, pos, kv)[0])
-        for i in reversed(range(len(LENGTHS))):
+        for i in reversed(range(len(lengths))):
             cache.add(i)
-        at = [0] * len(LENGTHS)
+        at = [0] * len(lengths)
         from distie_amd.parts import StepContext
-        for cut in CUTS:
+        for cut in cuts:
             entries, rows = [], []
             for i, n in enumerate(cut):
-                n = min(n, LENGTHS[i] - at[i])
+                n = min(n, lengths[i] - at[i])
                 if n >= 1:
                     cache.reserve(i, n)
                     entries.append(StepEntry(i, [0] * n, []))
