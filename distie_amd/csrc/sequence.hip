@@ -527,7 +527,7 @@ __global__ void causal_conv_bf16x8_kernel(const bf16_t* __restrict__ x, int64_t 
   if (cu_q[b + 1] - first == 1 && taps > 1) shift_state8(own, taps, c0, N, self);
 }
 
-// conv_rope_kv_write for bfloat16 products and caches, D, E and the number of pairs multiples of 8, DP == D or the
+// conv_rope_kv_write for steps of 32 rows and more, bfloat16 products and caches, D, E and the number of pairs multiples of 8, DP == D or the
 // places beyond D zeroed by eight. Blocks 0 .. T-1: q and k of one token (a thread turns eight pairs, or copies eight
 // single dimensions). The blocks behind them: v for 16 tokens each; a thread owns one channel of v and, where
 // the 16 tokens lie side by side in one page, writes their values as one run of 32 bytes (the cache keeps v with
@@ -545,7 +545,8 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
   const int N = H * D + (has_kv ? G * (D + E) : 0);
   if (static_cast<int>(blockIdx.x) >= T) {
     // ---- v: 16 tokens, one channel a thread
-    const int t0 = (static_cast<int>(blockIdx.x) - T) * VGROUP;
+    const int t0 = (static_cast<int>(blockIdx.x) - T) / G * VGROUP;
+    const int g = (static_cast<int>(blockIdx.x) - T) % G;
     const int n = min(VGROUP, T - t0);
     const int64_t slot0 = write ? slots[t0] : 0;
     bool together = write && n == VGROUP && block_size % 8 == 0 && slot0 % block_size % 8 == 0 &&
@@ -555,9 +556,8 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
       for (int k = 1; k < VGROUP; ++k) together = together && slots[min(t0 + k, T - 1)] == slot0 + k;
     }
     uint16_t* cache = reinterpret_cast<uint16_t*>(v_cache);
-    for (int item = threadIdx.x; item < G * E; item += blockDim.x) {
-      const int g = item / E, e = item % E;
-      const int c = (H + G) * D + item;
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+      const int c = (H + G) * D + g * E + e;
       float w[MAX_TAPS];
       for (int j = 0; j < taps; ++j) w[j] = to_float(weight[static_cast<int64_t>(c) * taps + j]);
       uint32_t bits[VGROUP];
@@ -741,6 +741,7 @@ scan_chunk_sums_kernel(const X* __restrict__ product, int64_t ld, const float* _
   __syncthreads();
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
   float acc[2][4][4] = {};
+#pragma unroll 4
   for (int j = 0; j < len; ++j) {
     const float4 v4 = *reinterpret_cast<const float4*>(Vs + j * 64 + 4 * tx);
     const float v[4] = {v4.x, v4.y, v4.z, v4.w};
@@ -843,6 +844,7 @@ scan_chunk_outputs_kernel(const X* __restrict__ product, int64_t ld, const float
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
   float s4[4][4] = {};
   if (tx <= ty) {
+#pragma unroll 8
     for (int d = 0; d < D; ++d) {
       const float4 q4 = *reinterpret_cast<const float4*>(Qt + d * SCAN_PAD + 4 * ty);
       const float4 k4 = *reinterpret_cast<const float4*>(Kt + d * SCAN_PAD + 4 * tx);
@@ -869,6 +871,7 @@ scan_chunk_outputs_kernel(const X* __restrict__ product, int64_t ld, const float
   }
   __syncthreads();
   float o[4][4] = {}, r[4][4] = {};
+#pragma unroll 8
   for (int d = 0; d < D; ++d) {
     const float4 q4 = *reinterpret_cast<const float4*>(Qt + d * SCAN_PAD + 4 * ty);
     const float4 t4 = *reinterpret_cast<const float4*>(Ss + d * 64 + 4 * tx);
@@ -879,6 +882,7 @@ scan_chunk_outputs_kernel(const X* __restrict__ product, int64_t ld, const float
       for (int b = 0; b < 4; ++b) r[a][b] += q[a] * t[b];
   }
   const int reach = min(len, 4 * ty + 4);
+#pragma unroll 4
   for (int j = 0; j < reach; ++j) {
     const float4 a4 = *reinterpret_cast<const float4*>(At + j * SCAN_PAD + 4 * ty);
     const float4 v4 = *reinterpret_cast<const float4*>(Vs + j * 64 + 4 * tx);
@@ -999,11 +1003,11 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
     return DISTIE_BAD_ARGUMENT;
   if (has_kv && write && (k_cache == nullptr || v_cache == nullptr || slots == nullptr)) return DISTIE_BAD_ARGUMENT;
   if (dtype == DISTIE_BF16 && (weight == nullptr || w_dtype == DISTIE_BF16) && (!write || cache_dtype == DISTIE_BF16) &&
-      D % 8 == 0 && E % 8 == 0 && DP % 8 == 0 && pairs % 8 == 0 && ld % 8 == 0 &&
+      T >= 32 && D % 8 == 0 && E % 8 == 0 && DP % 8 == 0 && pairs % 8 == 0 && ld % 8 == 0 &&
       reinterpret_cast<uintptr_t>(product) % 16 == 0 && reinterpret_cast<uintptr_t>(q_out) % 16 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(state) % 16 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0) {
     const int items = (has_kv ? H + G : H) * ((DP - pairs) / 8);
     const int threads8 = items > 128 ? 256 : (items > 64 ? 128 : 64);
-    const int v_blocks = has_kv && (write || taps > 1) ? (T + VGROUP - 1) / VGROUP : 0;
+    const int v_blocks = has_kv && (write || taps > 1) ? (T + VGROUP - 1) / VGROUP * G : 0;
     conv_rope_kv_write_bf16_kernel<<<T + v_blocks, threads8, 0, stream>>>(
         static_cast<const bf16_t*>(product), ld, static_cast<const bf16_t*>(weight), taps, state,
         static_cast<const float2*>(table), pairs, magnitude, static_cast<bf16_t*>(q_out), static_cast<bf16_t*>(k_cache),
