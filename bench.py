@@ -253,7 +253,13 @@ def design_run(args) -> int:
                       max_model_len=max(8192, tokens_per_request), tune_products=not args.no_tune)
             t_prefill = prefill_run(llm, prefill_tokens, TOKEN_BUDGET, DESIGN_VOCAB)
             step_s, _ = decode_run(llm, args.batch, context, args.steps, args.warmup, DESIGN_VOCAB, seed=1)
-            row[name] = {"weights_M": round(llm.model.weight_bytes() / (2 if args.dtype == "bf16" else 4) / 1e6, 1),
+            declared = 0
+            for spec in llm.model.param_specs().values():
+                count = 1
+                for n in spec.shape:
+                    count *= int(n)
+                declared += count
+            row[name] = {"weights_M": round(declared / 1e6, 1),
                          "prefill_tok_s": round(prefill_tokens / t_prefill, 1), "prefill_ms": round(t_prefill * 1e3, 3),
                          "decode_tok_s": round(args.batch / step_s, 1), "decode_ms_per_step": round(step_s * 1e3, 4)}
             llm.close()

@@ -1,4 +1,4 @@
-"""MI355X-native inference engine for the Qwen2 dense decoder."""
+"""MI355X-native inference engine for the Qwen2 dense decoder and the Musutar decoder."""
 
 from .config import EngineConfig
 from .engine import LLM, RequestOutput, StepEntry, Trace

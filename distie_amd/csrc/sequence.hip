@@ -2,7 +2,7 @@
 // several residual streams with learned read, mix and write weights; a short causal convolution over time
 // whose last inputs are a request's state; attention projections with such a convolution, a partial rotation
 // and the cache write behind it; a decayed outer-product state (linear attention) scanned over the tokens;
-// gates. Everything the card of such a design wants in 32-bit is float32 here in either precision: the
+// gates. What such designs keep in 32-bit is float32 here in either precision: the
 // streams, norm statistics, angles, the state and every sum that enters it.
 //
 // A step is a flattened batch: token t belongs to request token_request[t], whose new tokens are rows

@@ -283,3 +283,84 @@ def test_greedy_generation_through_the_scheduler(ops, folders):
                 ids.append(token)
         assert not llm.cache.live()
         llm.close()
+
+
+def test_random_model_folder_reads_back(tmp_path):
+    """`random-model` of the command line writes a folder that the loader takes, tensor for tensor as the design
+    names them."""
+    import json
+
+    from distie_amd import cli
+    from distie_amd.weights.safetensors_io import SafetensorsFile
+
+    (tmp_path / "config.json").write_text(json.dumps(PLAIN))
+    assert cli.main(["random-model", "--config-json", str(tmp_path / "config.json"), "--out", str(tmp_path / "m"),
+                     "--seed", "3", "--dtype", "bf16", "--std", "0.1"]) == 0
+    stored = SafetensorsFile(tmp_path / "m" / "model.safetensors")
+    assert {name: tuple(entry[1]) for name, entry in stored.index.items()} == mu.tensor_shapes(PLAIN)
+    stored.close()
+    llm = engine(tmp_path / "m", TorchOps(), "float32")
+    assert llm.step([StepEntry("a", [1, 2, 3], [2])]).shape == (1, PLAIN["vocab"])
+
+
+@pytest.mark.gpu
+def test_trace_runner_and_command_line(folders, tmp_path):
+    """The trace runner as a program (its own process, steps on standard input, four requests live, pages and
+    slots used again) and `generate` of the command line, on a Musutar model, against the plain implementation."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    import numpy as np
+
+    root = Path(__file__).resolve().parents[1]
+    folder, cfg, weights = folders["mixed"]
+    lengths = {"p": 70, "q": 33, "r": 64, "s": 5, "t": 90, "u": 41}
+    reqs = {r: mu.random_ids(cfg, n, 60 + n) for r, n in lengths.items()}
+    want = {r: mu.oracle(cfg, weights, ids) for r, ids in reqs.items()}
+    max_tokens = sum(-(-n // 64) * 64 for n in sorted(lengths.values())[-4:])
+    for dtype in ("float32", "bfloat16"):
+        out = tmp_path / dtype
+        proc = subprocess.Popen([sys.executable, str(root / "bin" / "trace_run"), "--model", str(folder), "--dtype", dtype,
+                                 "--out", str(out), "--max-tokens", str(max_tokens)],
+                                stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+        got, at = {r: [] for r in reqs}, {r: 0 for r in reqs}
+        waiting, live, step = list(reqs), [], 0
+        while waiting or live:
+            while waiting and len(live) < 4:
+                live.append(waiting.pop(0))
+            entries, end = [], []
+            for k, r in enumerate(live):
+                left = len(reqs[r]) - at[r]
+                n = min(left, 1 if left <= 8 else [13, 2, 30, 7][(step + k) % 4])
+                entries.append({"id": r, "tokens": reqs[r][at[r]:at[r] + n], "want": list(range(n))})
+                at[r] += n
+                if at[r] == len(reqs[r]):
+                    end.append(r)
+            proc.stdin.write(json.dumps({"step": step, "entries": entries, "end": end}) + "\n")
+            proc.stdin.flush()
+            assert proc.stdout.readline().strip() == f"done {step}"
+            rows = torch.from_numpy(np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(-1, cfg["vocab"]).copy())
+            row = 0
+            for e in entries:
+                got[e["id"]].append(rows[row:row + len(e["tokens"])])
+                row += len(e["tokens"])
+            live = [r for r in live if r not in end]
+            step += 1
+        proc.stdin.close()
+        assert proc.wait(timeout=60) == 0
+        for r in reqs:
+            check(torch.cat(got[r]), want[r], dtype, f"request {r} {dtype}")
+    prompts = [reqs["s"], reqs["q"][:9]]
+    (tmp_path / "prompts.json").write_text(json.dumps(prompts))
+    done = subprocess.run([sys.executable, "-m", "distie_amd.cli", "generate", "--model", str(folder), "--dtype", "fp32",
+                           "--prompts", str(tmp_path / "prompts.json"), "--max-new-tokens", "6", "--num-blocks", "32",
+                           "--out", str(tmp_path / "report.json")], cwd=str(root), capture_output=True, text=True, timeout=110)
+    assert done.returncode == 0, done.stderr
+    for prompt, record in zip(prompts, json.loads((tmp_path / "report.json").read_text())):
+        ids = list(prompt)
+        for token in record["token_ids"]:
+            logits = mu.oracle(cfg, weights, ids)[-1]
+            assert float(logits[token]) >= float(logits.max()) - 1e-3 * float(logits.abs().max())
+            ids.append(token)
