@@ -340,21 +340,36 @@ __global__ void sigmoid_gate_kernel(const X* __restrict__ x, int ldh, int E, con
   }
 }
 
-// out = x / sqrt(mean(x^2) + eps) * weight * sigmoid(gate): the norm over all heads together, then the gate
-template <typename W, typename G, typename O>
+// out = x / sqrt(mean(x^2) + eps) * weight * sigmoid(gate): the norm over all heads together, then the gate.
+// V channels a thread at a time (4: 16-byte loads of x, every load of a row under way before the sum).
+template <int V, typename W, typename G, typename O>
 __global__ void rmsnorm_gate_kernel(const float* __restrict__ x, const W* __restrict__ weight, float eps,
                                     const G* __restrict__ gates, int64_t ldg, O* __restrict__ out, int N) {
   __shared__ float scratch[16];
   const int64_t t = blockIdx.x;
   const float* row = x + t * N;
   float sq = 0.f;
-  for (int c = threadIdx.x; c < N; c += blockDim.x) sq += row[c] * row[c];
+  for (int c = V * threadIdx.x; c < N; c += V * blockDim.x) {
+    float v[V];
+    loadv<V>(row + c, v);
+#pragma unroll
+    for (int k = 0; k < V; ++k) sq += v[k] * v[k];
+  }
   sq = block_sum(sq, scratch);
   const float scale = 1.f / sqrtf(sq / N + eps);
-  for (int c = threadIdx.x; c < N; c += blockDim.x) {
-    float v = row[c] * scale * to_float(weight[c]);
-    if (gates != nullptr) v *= sigmoidf(to_float(gates[t * ldg + c]));
-    out[t * N + c] = from_float<O>(v);
+  for (int c = V * threadIdx.x; c < N; c += V * blockDim.x) {
+    float v[V], w[V];
+    loadv<V>(row + c, v);
+    loadv<V>(weight + c, w);
+#pragma unroll
+    for (int k = 0; k < V; ++k) v[k] *= scale * w[k];
+    if (gates != nullptr) {
+      float g[V];
+      loadv<V>(gates + t * ldg + c, g);
+#pragma unroll
+      for (int k = 0; k < V; ++k) v[k] *= sigmoidf(g[k]);
+    }
+    storev<V>(out + t * N + c, v);
   }
 }
 
@@ -705,6 +720,7 @@ __global__ void activation_bf16x8_kernel(const uint4* __restrict__ in, uint4* __
 // held in LDS; a chunk's table entry is {request, first row, rows, unused}.
 constexpr int SCAN_L = 64;
 constexpr int SCAN_PAD = 68;      // row stride of the transposed tiles: keeps 16-byte reads aligned
+constexpr int SCAN_BATCH = 8;     // loads a thread has under way while it fills a tile
 
 __device__ __forceinline__ void decay_powers(float* pw, float rate, int count) {
   if (threadIdx.x == 0) {
@@ -730,13 +746,31 @@ scan_chunk_sums_kernel(const X* __restrict__ product, int64_t ld, const float* _
   const int len = chunk.z;
   decay_powers(pw, decay[head], SCAN_L + 1);
   __syncthreads();
-  for (int idx = threadIdx.x; idx < SCAN_L * D; idx += 256) {
-    const int j = idx / D, d = idx % D;
-    Ks[idx] = j < len ? pw[len - 1 - j] * siluf(to_float(product[(row0 + j) * ld + (H + head) * D + d])) : 0.f;
-  }
-  for (int idx = threadIdx.x; idx < SCAN_L * 64; idx += 256) {
-    const int j = idx / 64, e = e0 + idx % 64;
-    Vs[idx] = (j < len && e < E) ? siluf(to_float(product[(row0 + j) * ld + 2 * H * D + head * E + e])) : 0.f;
+  // Tiles are filled row by row: lane = column, four rows a pass of the block, eight passes' loads under way at a
+  // time (a load that waits for the one before it costs a trip to memory each; no division by D in the loop).
+  const int col = threadIdx.x % 64, sub = threadIdx.x / 64;
+  for (int j0 = sub; j0 < SCAN_L; j0 += 4 * SCAN_BATCH) {
+    for (int d = col; d < D; d += 64) {
+      float k[SCAN_BATCH];
+#pragma unroll
+      for (int u = 0; u < SCAN_BATCH; ++u) {
+        const int j = j0 + 4 * u;
+        k[u] = j < len ? to_float(product[(row0 + j) * ld + (H + head) * D + d]) : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < SCAN_BATCH; ++u) {
+        const int j = j0 + 4 * u;
+        Ks[j * D + d] = j < len ? pw[len - 1 - j] * siluf(k[u]) : 0.f;
+      }
+    }
+    float v[SCAN_BATCH];
+#pragma unroll
+    for (int u = 0; u < SCAN_BATCH; ++u) {
+      const int j = j0 + 4 * u;
+      v[u] = (j < len && e0 + col < E) ? to_float(product[(row0 + j) * ld + 2 * H * D + head * E + e0 + col]) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < SCAN_BATCH; ++u) Vs[(j0 + 4 * u) * 64 + col] = siluf(v[u]);
   }
   __syncthreads();
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
@@ -764,11 +798,10 @@ scan_chunk_sums_kernel(const X* __restrict__ product, int64_t ld, const float* _
     for (int a = 0; a < 4; ++a) {
       const int d = 4 * ty + 64 * s + a;
       if (d >= D) continue;
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const int e = e0 + 4 * tx + b;
-        if (e < E) dst[static_cast<int64_t>(d) * E + e] = acc[s][a][b];
-      }
+      const int e = e0 + 4 * tx;                          // E is a multiple of 4: four columns are there or none
+      if (e < E)
+        *reinterpret_cast<float4*>(dst + static_cast<int64_t>(d) * E + e) =
+            float4{acc[s][a][0], acc[s][a][1], acc[s][a][2], acc[s][a][3]};
     }
 }
 
@@ -825,20 +858,32 @@ scan_chunk_outputs_kernel(const X* __restrict__ product, int64_t ld, const float
   const int64_t row0 = chunk.y;
   const int len = chunk.z;
   decay_powers(pw, decay[head], SCAN_L + 2);
-  for (int idx = threadIdx.x; idx < SCAN_L * D; idx += 256) {
-    const int j = idx / D, d = idx % D;
-    float q = 0.f, k = 0.f;
-    if (j < len) {
-      const X* row = product + (row0 + j) * ld;
-      q = siluf(to_float(row[head * D + d]));
-      k = siluf(to_float(row[(H + head) * D + d]));
+  const int col = threadIdx.x % 64, sub = threadIdx.x / 64;
+  for (int j0 = sub; j0 < SCAN_L; j0 += 4 * SCAN_BATCH) {
+    for (int d = col; d < D; d += 64) {
+      float q[SCAN_BATCH], k[SCAN_BATCH];
+#pragma unroll
+      for (int u = 0; u < SCAN_BATCH; ++u) {
+        const int j = j0 + 4 * u;
+        const X* row = product + (row0 + j) * ld;
+        q[u] = j < len ? to_float(row[head * D + d]) : 0.f;
+        k[u] = j < len ? to_float(row[(H + head) * D + d]) : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < SCAN_BATCH; ++u) {
+        const int j = j0 + 4 * u;
+        Qt[d * SCAN_PAD + j] = siluf(q[u]);
+        Kt[d * SCAN_PAD + j] = siluf(k[u]);
+      }
     }
-    Qt[d * SCAN_PAD + j] = q;
-    Kt[d * SCAN_PAD + j] = k;
-  }
-  for (int idx = threadIdx.x; idx < SCAN_L * 64; idx += 256) {
-    const int j = idx / 64, e = e0 + idx % 64;
-    Vs[idx] = (j < len && e < E) ? siluf(to_float(product[(row0 + j) * ld + 2 * H * D + head * E + e])) : 0.f;
+    float v[SCAN_BATCH];
+#pragma unroll
+    for (int u = 0; u < SCAN_BATCH; ++u) {
+      const int j = j0 + 4 * u;
+      v[u] = (j < len && e0 + col < E) ? to_float(product[(row0 + j) * ld + 2 * H * D + head * E + e0 + col]) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < SCAN_BATCH; ++u) Vs[(j0 + 4 * u) * 64 + col] = siluf(v[u]);
   }
   __syncthreads();
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
@@ -865,9 +910,16 @@ scan_chunk_outputs_kernel(const X* __restrict__ product, int64_t ld, const float
   __syncthreads();
   float* Ss = Kt;
   const float* src = scratch + (static_cast<int64_t>(c) * H + head) * D * E;
-  for (int idx = threadIdx.x; idx < D * 64; idx += 256) {
-    const int d = idx / 64, e = e0 + idx % 64;
-    Ss[idx] = e < E ? src[static_cast<int64_t>(d) * E + e] : 0.f;
+  for (int d0 = sub; d0 < D; d0 += 4 * SCAN_BATCH) {
+    float t[SCAN_BATCH];
+#pragma unroll
+    for (int u = 0; u < SCAN_BATCH; ++u) {
+      const int d = d0 + 4 * u;
+      t[u] = (d < D && e0 + col < E) ? src[static_cast<int64_t>(d) * E + e0 + col] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < SCAN_BATCH; ++u)
+      if (d0 + 4 * u < D) Ss[(d0 + 4 * u) * 64 + col] = t[u];
   }
   __syncthreads();
   float o[4][4] = {}, r[4][4] = {};
@@ -896,11 +948,11 @@ scan_chunk_outputs_kernel(const X* __restrict__ product, int64_t ld, const float
   for (int a = 0; a < 4; ++a) {
     const int i = 4 * ty + a;
     if (i >= len) continue;
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      const int e = e0 + 4 * tx + b;
-      if (e < E) out[((row0 + i) * H + head) * E + e] = o[a][b] + pw[i + 1] * r[a][b];
-    }
+    const int e = e0 + 4 * tx;
+    const float w = pw[i + 1];
+    if (e < E)
+      *reinterpret_cast<float4*>(out + ((row0 + i) * H + head) * E + e) =
+          float4{o[a][0] + w * r[a][0], o[a][1] + w * r[a][1], o[a][2] + w * r[a][2], o[a][3] + w * r[a][3]};
   }
 }
 
@@ -1051,11 +1103,22 @@ extern "C" int distie_rmsnorm_gate(const float* x, const void* weight, int w_dty
                                    int g_dtype, int64_t ldg, void* out, int out_dtype, int T, int N, hipStream_t stream) {
   if (T <= 0) return 0;
   if (N < 1 || (gates != nullptr && ldg < N)) return DISTIE_BAD_ARGUMENT;
-  const int threads = N >= 2048 ? 512 : (N >= 512 ? 256 : (N >= 128 ? 128 : 64));
   if (gates == nullptr) g_dtype = DISTIE_F32;
-  DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(g_dtype, G, DISTIE_DISPATCH(out_dtype, O,
-      rmsnorm_gate_kernel<W, G, O><<<T, threads, 0, stream>>>(
-          x, static_cast<const W*>(weight), eps, static_cast<const G*>(gates), ldg, static_cast<O*>(out), N))));
+  const bool wide = N % 8 == 0 && ldg % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(weight) % 16 == 0 && reinterpret_cast<uintptr_t>(gates) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const int per = wide ? N / 4 : N;
+  const int threads = per >= 1024 ? 1024 : (per >= 512 ? 512 : (per >= 256 ? 256 : (per >= 128 ? 128 : 64)));
+#define DISTIE_NORM_GATE(V)                                                                                  \
+  DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(g_dtype, G, DISTIE_DISPATCH(out_dtype, O,                      \
+      rmsnorm_gate_kernel<V, W, G, O><<<T, threads, 0, stream>>>(                                            \
+          x, static_cast<const W*>(weight), eps, static_cast<const G*>(gates), ldg, static_cast<O*>(out), N))))
+  if (wide) {
+    DISTIE_NORM_GATE(4);
+  } else {
+    DISTIE_NORM_GATE(1);
+  }
+#undef DISTIE_NORM_GATE
   return launch_status();
 }
 
