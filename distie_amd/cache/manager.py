@@ -21,7 +21,13 @@ tensor it names, a slab `[slots + 1, *shape]`; a request's rows are zeroed when 
 taken. The model of this engine has no such mixer, the slots exist all the same.
 
 A layer may hold several mixers (its block says which, by name): `requirements[l]` maps the name of
-each mixer of layer l to its declaration, and `layer(l)[name]` is that mixer's view.
+each mixer of layer l to its declaration, and `layer(l)[name]` is that mixer's view. A block may add
+entries of its own under other names (the last inputs of a convolution it runs in front of a mixer).
+
+A part that keeps pages and fixed state declares both (`CacheNeeds(paged, state)`): its view holds all
+tensors by name. `Borrowed(layer, name)` in place of pages: the part reads the pages of another layer's
+mixer, so its view holds that mixer's tensors and group; it owns no slab and takes no page, and the lender's
+declaration says how far back the pages must stay.
 """
 
 from __future__ import annotations

@@ -190,7 +190,8 @@ class Ops(abc.ABC):
         `init` (float32 [T, C]): the streams do not exist yet and all start as `init` (`streams` is None).
         `delta` (act [T, C], with `mix` float32 [S, S] indexed [from, to] and `write` float32 [S]): all streams
         at once from the old ones, x_j <- sum_s mix[s, j] x_s + write[j] * delta * sigmoid(gate) (`gate` act
-        [T, C] or a view with a row stride; None: no gate). `read` (float32 [S]): h = norm(sum_s read[s] x_s)
+        [T, C] or a view with a row stride; None: no gate). `delta` and `gate` may be what `linear` returned, in
+        whatever form. `read` (float32 [S]): h = norm(sum_s read[s] x_s)
         * norm_weight in `out_dtype`, from the updated streams; `norm` is "none" (h is the sum, float32 unless
         `out_dtype` says otherwise), "layer" ((u - mean) / sqrt(var + eps), var the mean of the squared deviations)
         or "rms" (u / sqrt(mean(u^2) + eps)). Statistics and sums in float32."""
