@@ -364,3 +364,24 @@ def test_trace_runner_and_command_line(folders, tmp_path):
             logits = mu.oracle(cfg, weights, ids)[-1]
             assert float(logits[token]) >= float(logits.max()) - 1e-3 * float(logits.abs().max())
             ids.append(token)
+
+
+def test_preemption_starts_the_state_over(ops, folders):
+    """So few pages that running requests are preempted and recomputed: their convolution inputs and decayed
+    states start from zero again, and every token still is the plain implementation's pick."""
+    folder, cfg, weights = folders["plain"]          # one of its layers keeps every key: the pages grow with the request
+    prompts = [mu.random_ids(cfg, n, seed=70 + n) for n in (20, 26, 17)]
+    block = 4 if ops.device.type == "cpu" else 16
+    new = 24 if block == 4 else 40
+    # as many pages as the longest request may hold by itself: three of them do not fit side by side
+    llm = engine(folder, ops, "float32", block_size=block, num_blocks=-(-(26 + new) // block) + 1, max_seqs=3, token_budget=32)
+    outs = llm.generate(prompts, SamplingParams(max_new_tokens=new))
+    assert sum(o.preemptions for o in outs) > 0, "the pool was not small enough to preempt anybody"
+    for prompt, out in zip(prompts, outs):
+        ids = list(prompt)
+        for token in out.token_ids:
+            logits = mu.oracle(cfg, weights, ids)[-1]
+            assert float(logits[token]) >= float(logits.max()) - 1e-3 * float(logits.abs().max())
+            ids.append(token)
+    llm.cache.check()
+    assert not llm.cache.live()
