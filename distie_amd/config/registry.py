@@ -11,6 +11,7 @@ from __future__ import annotations
 from typing import Any, Dict, Mapping
 
 from .model_config import ConfigError, ModelSpec, Qwen2Config, read_config_json
+from .duparax_config import DuparaxConfig
 from .musutar_config import MusutarConfig
 
 _ARCHITECTURES: Dict[str, Any] = {}
@@ -44,8 +45,23 @@ def config_from_dict(config_json: Mapping[str, Any]):
 
 
 def load_model_config(model_dir):
-    """The typed config of the model folder `model_dir`."""
-    return config_from_dict(read_config_json(model_dir))
+    """The typed config of the model folder `model_dir`. A design that leaves a size to the shape of a tensor
+    (its config class has `with_tensor_shapes`) gets the names and shapes of the folder's tensors, read from the
+    files' headers."""
+    config = config_from_dict(read_config_json(model_dir))
+    if hasattr(config, "with_tensor_shapes"):
+        from ..weights.safetensors_io import SafetensorsFile, model_files   # local import: weights read configs too
+
+        shapes = {}
+        files = model_files(model_dir)
+        for path in set(files.values()):
+            source = SafetensorsFile(path)
+            try:
+                shapes.update({name: tuple(entry[1]) for name, entry in source.index.items()})
+            finally:
+                source.close()
+        config = config.with_tensor_shapes(shapes)
+    return config
 
 
 def model_spec_from_dir(model_dir) -> ModelSpec:
@@ -54,3 +70,4 @@ def model_spec_from_dir(model_dir) -> ModelSpec:
 
 register_architecture(Qwen2Config.architecture, Qwen2Config)
 register_architecture(MusutarConfig.architecture, MusutarConfig)
+register_architecture(DuparaxConfig.architecture, DuparaxConfig)

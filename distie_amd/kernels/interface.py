@@ -159,8 +159,9 @@ class Ops(abc.ABC):
         return self.silu_mul(self.linear(x, gate_up_weight))
 
     @abc.abstractmethod
-    def linear_f32out(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-        """As `linear` without bias, result in float32 (the logits)."""
+    def linear_f32out(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                      scale: float = 1.0) -> torch.Tensor:
+        """As `linear`, result in float32 and not rounded (the logits; what enters a recurrence), times `scale`."""
 
     @abc.abstractmethod
     def rope_kv_write(self, qkv: torch.Tensor, meta: BatchMeta, group: int, k_cache: torch.Tensor,
@@ -204,8 +205,9 @@ class Ops(abc.ABC):
                                eps=eps, out_dtype=out_dtype)[1]
 
     def causal_conv(self, x: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor], meta: BatchMeta,
-                    residual: bool = False) -> torch.Tensor:
-        """x act [T, N], weight [N, taps] -> y_t = (x_t if residual) + sum_j weight[:, j] * x_(t - taps + 1 + j)
+                    residual: bool = False, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x act [T, N] (or a view of columns with a row stride), weight [N, taps], bias float32 [N] or None
+        -> y_t = bias + (x_t if residual) + sum_j weight[:, j] * x_(t - taps + 1 + j)
         within each request; what lies before the step's rows comes from `state` (float32 [slots + 1, taps - 1, N],
         the request's last taps - 1 inputs, oldest first, rows by `meta.state_slots`), which is moved on to the
         end of the step's rows. Sums in float32, in the order of j."""
@@ -215,7 +217,8 @@ class Ops(abc.ABC):
                            state: Optional[torch.Tensor], meta: BatchMeta, group: int,
                            k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                            inv_freq: Optional[torch.Tensor], magnitude: float, num_heads: int, num_kv_heads: int,
-                           dim: int, value_dim: int, padded_dim: int, has_kv: bool, write: bool) -> torch.Tensor:
+                           dim: int, value_dim: int, padded_dim: int, has_kv: bool, write: bool,
+                           q_temp=None) -> torch.Tensor:
         """Behind attention's stacked projection. The first columns of `product` (act [T, W]) are q (num_heads x
         dim) and, if `has_kv`, k (num_kv_heads x dim) and v (num_kv_heads x value_dim); further columns are left
         alone. Each of these channels goes through `causal_conv` (no residual; `conv_weight` [channels, taps],
@@ -223,13 +226,15 @@ class Ops(abc.ABC):
         are rotated by the token's position (pair (i, i + len(inv_freq)); cosine and sine both times
         `magnitude`), and, if `write`, k and v go to the token's slot of k_cache [pages, KH, P, padded_dim] /
         v_cache [pages, KH, padded_dim, P]. Returns q as act [T, num_heads * padded_dim], zeros beyond `dim`:
-        what `paged_attention` reads with a head size of `padded_dim`."""
+        what `paged_attention` reads with a head size of `padded_dim`.
+        `q_temp` = (coef, every): a query temperature by position, q of the token at position p is multiplied by
+        1 + coef * ln(floor((p + 1) / every) + 1), computed in float32 (None: none)."""
         raise NotImplementedError(f"{type(self).__name__} has no convolution over time")
 
     def sigmoid_gate(self, x: torch.Tensor, num_heads: int, head_stride: int, width: int,
                      gates: torch.Tensor) -> torch.Tensor:
         """x act [T, num_heads * head_stride], of which the first `width` of every head count; gates act
-        [T, num_heads * width] (or a view with a row stride) -> x * sigmoid(gates), act [T, num_heads * width]."""
+        [T, num_heads * width] (or a view with a row stride) -> x * sigmoid(gates), act [T, num_heads * width]. `gates` None: the kept columns as they are."""
         raise NotImplementedError(f"{type(self).__name__} has no gates")
 
     def decay_scan(self, product: torch.Tensor, state: torch.Tensor, decay: torch.Tensor, meta: BatchMeta,
@@ -242,10 +247,71 @@ class Ops(abc.ABC):
         raise NotImplementedError(f"{type(self).__name__} has no decayed state")
 
     def rmsnorm_gate(self, x: torch.Tensor, weight: torch.Tensor, eps: float, gates: Optional[torch.Tensor],
-                     out_dtype) -> torch.Tensor:
+                     out_dtype, group: Optional[int] = None, gate: str = "sigmoid") -> torch.Tensor:
         """float32 [T, N] -> x / sqrt(mean(x^2) + eps) * weight * sigmoid(gates) in `out_dtype` (gates act [T, N]
-        or a view with a row stride; None: no gate)."""
+        or a view with a row stride; None: no gate). `group`: the mean is taken over every run of `group` columns
+        by itself (a head), and `weight` [group] is the same for all of them; None: over all N, weight [N].
+        `gate`: "sigmoid" or "silu" (times gates * sigmoid(gates))."""
         raise NotImplementedError(f"{type(self).__name__} has no gated norm")
+
+    # ---- sums of normed sub-layer outputs, states with a decay of their own for every channel and token, routed
+    # ---- feed-forwards. As above: an implementation that serves no model with them may leave them out.
+    def normed_sum(self, terms, weights, eps: float, scale: float):
+        """scale * sum_i rmsnorm(terms[i]) * weights[i] -> float32 [T, C] (mixers side by side on one input, each
+        result normed over the model width before they are added). `terms`: act [T, C] each, or what `linear`
+        returned; `weights` float32 [C] each. An implementation may hand out a value that only `add_normed`,
+        `add_normed_rmsnorm` and `dense` read."""
+        raise NotImplementedError(f"{type(self).__name__} has no sum of normed terms")
+
+    def add_normed(self, residual: torch.Tensor, delta, weight: torch.Tensor, eps: float) -> None:
+        """residual (float32 [T, C], in place) += rmsnorm(delta) * weight: a sub-layer's result with a norm behind
+        it. `delta`: act [T, C], what `linear` returned, or what `normed_sum` returned."""
+        raise NotImplementedError(f"{type(self).__name__} has no norm behind a sub-layer")
+
+    def add_normed_rmsnorm(self, residual: torch.Tensor, delta, post_weight: torch.Tensor, post_eps: float,
+                           weight: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+        """`add_normed`, then rmsnorm(residual) * weight in `out_dtype`; an implementation may fuse the two."""
+        self.add_normed(residual, delta, post_weight, post_eps)
+        return self.rmsnorm(residual, weight, eps, out_dtype)
+
+    def gated_decay_scan(self, product: torch.Tensor, decay_logits: torch.Tensor, state: torch.Tensor, meta: BatchMeta,
+                         num_heads: int, dim: int, value_dim: int, q_scale: float, tau: float) -> torch.Tensor:
+        """Linear attention whose state decays by a factor of its own for every key channel and token: with q
+        (num_heads x dim, times `q_scale`), k (num_heads x dim) and v (num_heads x value_dim) from the first columns
+        of `product` (act [T, W]) and alpha = sigmoid(decay_logits)^(1 / tau) (decay_logits float32 [T, num_heads *
+        dim]), per head S <- diag(alpha) S + k v^T (alpha scales the rows of S, one a key channel) and o = S^T q.
+        `state` float32 [slots + 1, num_heads, dim, value_dim] (rows by `meta.state_slots`) is read and left as
+        the step's last row leaves it. -> float32 [T, num_heads * value_dim]; decay, state and sums in float32."""
+        raise NotImplementedError(f"{type(self).__name__} has no gated decayed state")
+
+    def lru_gates(self, u: torch.Tensor, recur_weight: torch.Tensor, recur_bias: torch.Tensor,
+                  input_weight: torch.Tensor, input_bias: torch.Tensor, lam: torch.Tensor, rate: float):
+        """The coefficients of a real-gated linear recurrent unit. u act [T, R] in B equal parts; the gates'
+        weights are block-diagonal, [B, R/B, R/B] with each block [out, in], biases float32 [B, R/B]:
+        r = sigmoid(W_r u + b_r), i = sigmoid(W_i u + b_i), a = exp(-rate * r * softplus(lam)) (lam float32 [R]),
+        x = sqrt(1 - a^2) * i * u -> (a, x), float32 [T, R] each; sums and everything behind them in float32."""
+        raise NotImplementedError(f"{type(self).__name__} has no gated linear recurrent unit")
+
+    def lru_scan(self, a: torch.Tensor, x: torch.Tensor, state: torch.Tensor, meta: BatchMeta,
+                 mul: Optional[torch.Tensor], mul_act: Optional[str], out_dtype) -> torch.Tensor:
+        """h_t = a_t * h_(t-1) + x_t for every channel, over each request's rows in order (a, x float32 [T, R]);
+        `state` float32 [slots + 1, R] (rows by `meta.state_slots`) holds h in front of the step and is left as the
+        last row leaves it. -> h * act(mul) in `out_dtype` (`mul` act [T, R] or a view with a row stride, `mul_act`
+        one of `activation`'s names or None for mul itself; `mul` None: h)."""
+        raise NotImplementedError(f"{type(self).__name__} has no gated linear recurrent unit")
+
+    def route_topk(self, x, weight: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+        """The router of a mixture of experts: z = weight x + bias in float32 (x act [T, C], weight [E, C], bias
+        float32 [E]); for every row the `top` largest z (the lower index among equals) and softmax over those alone
+        -> (experts int32 [T, top], their weights float32 [T, top]), largest first."""
+        raise NotImplementedError(f"{type(self).__name__} has no router")
+
+    def route_scale(self, hidden: torch.Tensor, experts: torch.Tensor, gates: torch.Tensor, num_experts: int,
+                    width: int) -> torch.Tensor:
+        """hidden act [T, num_experts * width + more] (in place): the columns of expert e, [e * width, (e + 1) *
+        width), times the row's weight for e, or zero if the row did not choose e; columns beyond the experts' (a
+        part that every row uses) stay. -> hidden."""
+        raise NotImplementedError(f"{type(self).__name__} has no routed feed-forward")
 
     def activation(self, x, kind: str) -> torch.Tensor:
         """Element by element on act [T, N]: "relu2" (the square of max(x, 0)), "silu", "gelu_tanh", "relu"."""

@@ -156,5 +156,58 @@ class HyperConnections(Block):
         stream.lanes["pending"] = (y, gate, self.mix[2], self.write[2])
 
 
+class SandwichResidual(Block):
+    """A norm in front of each sub-layer and another behind it, the second inside the residual branch:
+
+        x <- x + mixer_post_norm(mixer(mixer_norm(x)));   x <- x + feed_forward_post_norm(feed_forward(feed_forward_norm(x)))
+
+    All four are RMS norms. A layer may have no feed-forward. A sub-layer's result stays pending with the norm that
+    belongs behind it; the norm in front of the next sub-layer (or the model's last norm) adds it while it reads the
+    residual (`Ops.add_normed_rmsnorm`: one kernel between two sub-layers)."""
+
+    CHILDREN = {"mixer_norm": "norm", "mixer": "mixer", "mixer_post_norm": "norm",
+                "feed_forward_norm": "norm", "feed_forward": "feed_forward", "feed_forward_post_norm": "norm"}
+    OPTIONAL = ("feed_forward_norm", "feed_forward", "feed_forward_post_norm")
+
+    def __init__(self, spec, parts) -> None:
+        super().__init__(spec, parts)
+        present = [self.feed_forward is None, self.feed_forward_norm is None, self.feed_forward_post_norm is None]
+        if any(present) and not all(present):
+            raise ValueError("a feed-forward and its two norms come together")
+        for norm in (self.mixer_norm, self.mixer_post_norm, self.feed_forward_norm, self.feed_forward_post_norm):
+            if norm is not None and getattr(norm, "fused_kind", None) != "rms":
+                raise ValueError("the sandwich arrangement takes RMS norms")
+
+    @staticmethod
+    def _settle(ops, stream: ResidualStream) -> None:
+        lanes, stream.lanes = stream.lanes, None
+        if lanes and lanes.get("pending") is not None:
+            delta, post = lanes["pending"]
+            ops.add_normed(stream.hidden, delta, post.weight, post.eps)
+
+    def _enter(self, ops, stream: ResidualStream, norm, act_dtype):
+        """Add what is pending, through the norm behind its sub-layer, and norm the residual for the next one."""
+        if stream.pending is not None:
+            raise ValueError("the sandwich arrangement starts from a residual with nothing pending on it")
+        pending = stream.lanes.get("pending") if stream.lanes else None
+        if pending is None:
+            return norm.apply(ops, stream.hidden, act_dtype)
+        delta, post = pending
+        stream.lanes["pending"] = None
+        return ops.add_normed_rmsnorm(stream.hidden, delta, post.weight, post.eps, norm.weight, norm.eps, act_dtype)
+
+    def forward(self, ops, stream: ResidualStream, ctx: StepContext, cache, writes_cache: bool) -> None:
+        h = self._enter(ops, stream, self.mixer_norm, ctx.act_dtype)
+        y = self.mixer.forward(ops, h, ctx, cache["mixer"], writes_cache)
+        stream.lanes = {"pending": (y, self.mixer_post_norm)}
+        stream.settle = self._settle
+        if self.feed_forward is None:
+            return
+        h = self._enter(ops, stream, self.feed_forward_norm, ctx.act_dtype)
+        y = self.feed_forward.forward(ops, h, ctx)
+        stream.lanes["pending"] = (y, self.feed_forward_post_norm)
+
+
 register_part("block", "prenorm_residual", PreNormResidual)
+register_part("block", "sandwich_residual", SandwichResidual)
 register_part("block", "hyper_connections", HyperConnections)

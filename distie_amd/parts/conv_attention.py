@@ -7,12 +7,15 @@
   its frequencies and the factor on cosine and sine);
 * keys of size `head_dim` and values of another size `value_dim`;
 * an output gate: the concatenated heads times sigmoid(W_g h), h being the mixer's input, before the output projection;
+* biases on q, k and v (`bias`: tensors `<q|k|v>.b`, added in the projection);
+* a query temperature by position (`q_temp` = {coef, every}): q at position p is multiplied by
+  1 + coef * ln(floor((p + 1) / every) + 1), in float32, so that later queries weigh their keys more sharply;
 * keys and values borrowed from an earlier layer (`kv_from`): such a layer has no k or v tensors; it reads the other
   layer's cache (keys as they lie there, convolved and rotated; values convolved) with queries, window and everything
   else of its own. The lending layer must keep its pages for as long as a borrower looks back (`keep`).
 
 score = q . k * scale over the keys j with 0 <= i - j < window (all j <= i without a window), ordinary softmax.
-No biases. The projections (and the gate's) are one matrix product: their weights are stacked at load. The kernels
+The projections (and the gate's) are one matrix product: their weights are stacked at load. The kernels
 work on one head size: max(head_dim, value_dim) rounded up to what the matrix-core kernels take, with zeros in the
 places beyond (they add nothing to a score and come out as zeros that are dropped).
 """
@@ -53,6 +56,11 @@ class ConvGatedAttention(Mixer):
         self.scale = float(p.get("scale", self.head_dim ** -0.5))
         self.output_gate = bool(p.get("output_gate", True))
         self.kv_from = p.get("kv_from")
+        self.bias = bool(p.get("bias", False))
+        temp = p.get("q_temp")
+        self.q_temp = (float(temp["coef"]), int(temp["every"])) if temp else None
+        if self.q_temp is not None and self.q_temp[1] < 1:
+            raise ValueError("q_temp.every must be >= 1")
         if self.num_heads % self.num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         self.position = build_part("position", p.get("position") or PartSpec("none"))
@@ -61,7 +69,7 @@ class ConvGatedAttention(Mixer):
         q, k, v = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim, self.num_kv_heads * self.value_dim
         self.conv_channels = q + (k + v if self.has_kv else 0)
         self.gate_width = self.num_heads * self.value_dim
-        self.in_weight = self.conv_weight = self.out_weight = None
+        self.in_weight = self.in_bias = self.conv_weight = self.out_weight = None
 
     def _projections(self):
         q, k, v = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim, self.num_kv_heads * self.value_dim
@@ -78,6 +86,9 @@ class ConvGatedAttention(Mixer):
         specs = {}
         for name, rows in self._projections():
             specs[name] = ParamSpec((rows, self.hidden_size))
+        if self.bias:
+            for name, rows in self._projections():
+                specs[name + ".b"] = ParamSpec((rows,))
         if self.conv_taps:
             for name, rows in self._projections():
                 specs[name + ".conv"] = ParamSpec((rows, self.conv_taps))
@@ -90,6 +101,11 @@ class ConvGatedAttention(Mixer):
         stacked = [tensors[name] for name, _ in self._projections()] + ([tensors["g"]] if self.output_gate else [])
         dtype = torch.float32 if any(t.dtype == torch.float32 for t in stacked) else stacked[0].dtype
         self.in_weight = torch.cat([t.to(dtype) for t in stacked], dim=0).contiguous()
+        if self.bias:
+            biases = [tensors[name + ".b"].float() for name, _ in self._projections()]
+            if self.output_gate:
+                biases.append(torch.zeros(self.gate_width, dtype=torch.float32, device=biases[0].device))
+            self.in_bias = torch.cat(biases).contiguous()
         if self.conv_taps:
             self.conv_weight = torch.cat([tensors[name + ".conv"] for name, _ in self._projections()], dim=0).contiguous()
         self.out_weight = tensors["o"].contiguous()
@@ -104,20 +120,20 @@ class ConvGatedAttention(Mixer):
         return classes[min(bisect.bisect_left(classes, longest), len(classes) - 1)]
 
     def forward(self, ops, x, ctx, cache, writes_cache: bool):
-        product = ops.dense(ops.linear(x, self.in_weight))
+        product = ops.dense(ops.linear(x, self.in_weight, self.in_bias))
         k_cache, v_cache = cache["k"], cache["v"]
         state = cache["conv"] if self.conv_taps > 1 else None
         q = ops.conv_rope_kv_write(product, self.conv_weight, state, ctx.meta, cache.group, k_cache, v_cache,
                                    self.position.rotary(), self.position.rotary_magnitude(), self.num_heads,
                                    self.num_kv_heads, self.head_dim, self.value_dim, self.padded_dim, self.has_kv,
-                                   writes_cache and self.has_kv)
+                                   writes_cache and self.has_kv, self.q_temp)
         mixed = ops.paged_attention(q, ctx.meta, cache.group, k_cache, v_cache, self.num_heads, self.num_kv_heads,
                                     self.padded_dim, self.scale, self.window)
         if self.output_gate:
             gates = product[:, self.conv_channels:self.conv_channels + self.gate_width]
             mixed = ops.sigmoid_gate(mixed, self.num_heads, self.padded_dim, self.value_dim, gates)
         elif self.padded_dim != self.value_dim:
-            raise NotImplementedError("values narrower than the kernels' head size need the output gate's kernel")
+            mixed = ops.sigmoid_gate(mixed, self.num_heads, self.padded_dim, self.value_dim, None)
         return ops.linear(mixed, self.out_weight)
 
 

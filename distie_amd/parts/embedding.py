@@ -33,6 +33,7 @@ class LinearHead(Head):
         self.hidden_size = int(spec.params["hidden_size"])
         self.tied_to = spec.params.get("tied_to")        # full name of the tensor to share, or None
         self.weight_name = spec.params.get("weight_name", "weight")
+        self.scale = float(spec.params.get("scale", 1.0))       # what the logits are multiplied by
         self.weight = None
 
     def param_specs(self):
@@ -51,7 +52,9 @@ class LinearHead(Head):
         ops.prepare_linear(self.weight, role="head")
 
     def forward(self, ops, normed):
-        return ops.linear_f32out(normed, self.weight)
+        if self.scale == 1.0:
+            return ops.linear_f32out(normed, self.weight)
+        return ops.linear_f32out(normed, self.weight, None, self.scale)
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)

@@ -62,4 +62,72 @@ class DecayLinearAttention(Mixer):
         return ops.linear(normed, self.out_weight)
 
 
+class GatedLinearAttention(Mixer):
+    """Linear attention whose state forgets channel by channel, by a gate computed from the token.
+
+    q = W_q h * dim^(-1/2), k = W_k h (heads x dim), v = W_v h (heads x value_dim), no activation. A decay for
+    every key channel, alpha = sigmoid(z)^(1 / tau) with z = W_a2 (W_a1 h) + b_a2 (a projection through `decay_rank`
+    dimensions), laid out like k. Per head
+
+        S_t = diag(alpha_t) S_(t-1) + k_t v_t^T,        o_t = S_t^T q_t.
+
+    Every head's o goes through an RMS norm over its value_dim columns (weight `norm` [value_dim], the same for all
+    heads), the heads side by side are multiplied by silu(W_g h) and projected by W_o. The state starts at zero and
+    is float32 [heads, dim, value_dim] for each request; the decay (sigmoid, logarithm, power), the products k v^T
+    and S^T q and the norm are float32 in either precision; z is not rounded on its way into the recurrence."""
+
+    def __init__(self, spec: PartSpec) -> None:
+        super().__init__(spec)
+        p = spec.params
+        self.hidden_size = int(p["hidden_size"])
+        self.num_heads = int(p["num_heads"])
+        self.head_dim = int(p["head_dim"])
+        self.value_dim = int(p.get("value_dim") or self.head_dim)
+        self.decay_rank = int(p["decay_rank"])
+        self.tau = float(p["tau"])
+        self.eps = float(p["eps"])
+        if not self.tau > 0:
+            raise ValueError("tau must be positive")
+        self.q_scale = float(p.get("q_scale", self.head_dim ** -0.5))
+        self.in_weight = self.low_weight = self.up_weight = self.up_bias = self.out_weight = self.norm_weight = None
+
+    def cache_requirement(self):
+        return FixedState.of((self.num_heads, self.head_dim, self.value_dim))
+
+    def param_specs(self):
+        qk, v = self.num_heads * self.head_dim, self.num_heads * self.value_dim
+        return {"q": ParamSpec((qk, self.hidden_size)), "k": ParamSpec((qk, self.hidden_size)),
+                "v": ParamSpec((v, self.hidden_size)), "g": ParamSpec((v, self.hidden_size)),
+                "o": ParamSpec((self.hidden_size, v)), "norm": ParamSpec((self.value_dim,), "ones"),
+                "a1": ParamSpec((self.decay_rank, self.hidden_size)), "a2": ParamSpec((qk, self.decay_rank)),
+                "a2.b": ParamSpec((qk,))}
+
+    def load(self, tensors) -> None:
+        stacked = [tensors[name] for name in "qkvg"]
+        dtype = torch.float32 if any(t.dtype == torch.float32 for t in stacked) else stacked[0].dtype
+        self.in_weight = torch.cat([t.to(dtype) for t in stacked], dim=0).contiguous()
+        self.low_weight = tensors["a1"].contiguous()
+        self.up_weight = tensors["a2"].contiguous()
+        self.up_bias = tensors["a2.b"].float().contiguous()
+        self.out_weight = tensors["o"].contiguous()
+        self.norm_weight = tensors["norm"].contiguous()
+
+    def prepare(self, ops) -> None:
+        ops.prepare_linear(self.in_weight, role="qkv")
+        ops.prepare_linear(self.out_weight, role="attn_out")
+
+    def forward(self, ops, x, ctx, cache, writes_cache: bool):
+        product = ops.dense(ops.linear(x, self.in_weight))
+        low = ops.dense(ops.linear(x, self.low_weight))
+        logits = ops.linear_f32out(low, self.up_weight, self.up_bias)
+        mixed = ops.gated_decay_scan(product, logits, cache["state"], ctx.meta, self.num_heads, self.head_dim,
+                                     self.value_dim, self.q_scale, self.tau)
+        first = self.num_heads * (2 * self.head_dim + self.value_dim)
+        gates = product[:, first:first + self.num_heads * self.value_dim]
+        normed = ops.rmsnorm_gate(mixed, self.norm_weight, self.eps, gates, ctx.act_dtype, group=self.value_dim,
+                                  gate="silu")
+        return ops.linear(normed, self.out_weight)
+
+
 register_part("mixer", "decay_linear_attention", DecayLinearAttention)
+register_part("mixer", "gated_linear_attention", GatedLinearAttention)

@@ -16,13 +16,14 @@ class RMSNorm(Norm):
         super().__init__(spec)
         self.size = int(spec.params["size"])
         self.eps = float(spec.params["eps"])
+        self.weight_name = spec.params.get("weight_name", "weight")      # the tensor's name behind the prefix
         self.weight = None
 
     def param_specs(self):
-        return {"weight": ParamSpec((self.size,), "ones")}
+        return {self.weight_name: ParamSpec((self.size,), "ones")}
 
     def load(self, tensors) -> None:
-        self.weight = tensors["weight"].contiguous()
+        self.weight = tensors[self.weight_name].contiguous()
 
     def apply(self, ops, x, out_dtype):
         return ops.rmsnorm(x, self.weight, self.eps, out_dtype)

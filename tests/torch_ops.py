@@ -35,8 +35,11 @@ class TorchOps(Ops):
             y = y + bias.float()
         return y.to(x.dtype)
 
-    def linear_f32out(self, x, weight):
-        return x.float() @ weight.float().T
+    def linear_f32out(self, x, weight, bias=None, scale=1.0):
+        y = x.float() @ weight.float().T
+        if bias is not None:
+            y = y + bias.float()
+        return y * scale if scale != 1.0 else y
 
     def rope_kv_write(self, qkv, meta, group, k_cache, v_cache, inv_freq, num_heads, num_kv_heads,
                       head_dim, write):
@@ -133,11 +136,12 @@ class TorchOps(Ops):
             out += x.float()
         return out
 
-    def causal_conv(self, x, weight, state, meta, residual=False):
-        return self._conv(x, weight, state, meta, residual).to(x.dtype)
+    def causal_conv(self, x, weight, state, meta, residual=False, bias=None):
+        y = self._conv(x, weight, state, meta, residual)
+        return (y if bias is None else y + bias.float()).to(x.dtype)
 
     def conv_rope_kv_write(self, product, conv_weight, state, meta, group, k_cache, v_cache, inv_freq, magnitude,
-                           num_heads, num_kv_heads, dim, value_dim, padded_dim, has_kv, write):
+                           num_heads, num_kv_heads, dim, value_dim, padded_dim, has_kv, write, q_temp=None):
         T = product.shape[0]
         channels = num_heads * dim + (num_kv_heads * (dim + value_dim) if has_kv else 0)
         u = product[:, :channels]
@@ -154,10 +158,14 @@ class TorchOps(Ops):
             return torch.cat([a * cos - b * sin, b * cos + a * sin, x[..., 2 * pairs:]], -1)
 
         q = torch.zeros(T, num_heads, padded_dim, dtype=torch.float32, device=product.device)
-        q[..., :dim] = turned(u[:, :num_heads * dim].view(T, num_heads, dim))
+        q[..., :dim] = turned(u[:, :num_heads * dim].reshape(T, num_heads, dim))
+        if q_temp is not None:
+            coef, every = q_temp
+            steps = torch.div(meta.positions.long() + 1, int(every), rounding_mode="floor")
+            q = q * (1.0 + float(coef) * torch.log(steps.float() + 1.0))[:, None, None]
         if has_kv and write:
-            k = turned(u[:, num_heads * dim:(num_heads + num_kv_heads) * dim].view(T, num_kv_heads, dim))
-            v = u[:, (num_heads + num_kv_heads) * dim:].view(T, num_kv_heads, value_dim)
+            k = turned(u[:, num_heads * dim:(num_heads + num_kv_heads) * dim].reshape(T, num_kv_heads, dim))
+            v = u[:, (num_heads + num_kv_heads) * dim:].reshape(T, num_kv_heads, value_dim)
             P = k_cache.shape[2]
             slots = meta.groups[group].slots.long()
             k_cache[slots // P, :, slots % P, :dim] = k.to(k_cache.dtype)
@@ -167,7 +175,7 @@ class TorchOps(Ops):
     def sigmoid_gate(self, x, num_heads, head_stride, width, gates):
         T = x.shape[0]
         kept = x.view(T, num_heads, head_stride)[..., :width].reshape(T, num_heads * width).float()
-        return (kept * torch.sigmoid(gates.float())).to(x.dtype)
+        return (kept if gates is None else kept * torch.sigmoid(gates.float())).to(x.dtype)
 
     def decay_scan(self, product, state, decay, meta, num_heads, dim, value_dim):
         T = product.shape[0]
@@ -186,11 +194,80 @@ class TorchOps(Ops):
             state[slots[b]] = s
         return out.view(T, num_heads * value_dim)
 
-    def rmsnorm_gate(self, x, weight, eps, gates, out_dtype):
-        y = x / torch.sqrt((x ** 2).mean(-1, keepdim=True) + eps) * weight.float()
+    def rmsnorm_gate(self, x, weight, eps, gates, out_dtype, group=None, gate="sigmoid"):
+        T, N = x.shape
+        v = x.view(T, N // group, group) if group else x
+        y = (v / torch.sqrt((v ** 2).mean(-1, keepdim=True) + eps) * weight.float()).reshape(T, N)
         if gates is not None:
-            y = y * torch.sigmoid(gates.float())
+            g = gates.float()
+            y = y * (torch.sigmoid(g) if gate == "sigmoid" else g * torch.sigmoid(g))
         return y.to(out_dtype)
+
+    # ---- sums of normed terms, states with their own decays, routers
+    @staticmethod
+    def _rms(x, weight, eps):
+        x = x.float()
+        return x / torch.sqrt((x ** 2).mean(-1, keepdim=True) + eps) * weight.float()
+
+    def normed_sum(self, terms, weights, eps, scale):
+        return scale * sum(self._rms(t, w, eps) for t, w in zip(terms, weights))
+
+    def add_normed(self, residual, delta, weight, eps):
+        residual += self._rms(delta, weight, eps)
+
+    def gated_decay_scan(self, product, decay_logits, state, meta, num_heads, dim, value_dim, q_scale, tau):
+        T = product.shape[0]
+        H, D, E = num_heads, dim, value_dim
+        q = product[:, :H * D].float().view(T, H, D) * q_scale
+        k = product[:, H * D:2 * H * D].float().view(T, H, D)
+        v = product[:, 2 * H * D:H * (2 * D + E)].float().view(T, H, E)
+        alpha = torch.exp(torch.nn.functional.logsigmoid(decay_logits.float()) / tau).view(T, H, D)
+        out = torch.zeros(T, H, E, dtype=torch.float32, device=product.device)
+        cu, slots = meta.cu_q.tolist(), meta.state_slots.tolist()
+        for b in range(meta.num_requests):
+            s = state[slots[b]]
+            for t in range(cu[b], cu[b + 1]):
+                s = alpha[t][:, :, None] * s + k[t][:, :, None] * v[t][:, None, :]
+                out[t] = torch.einsum("hde,hd->he", s, q[t])
+            state[slots[b]] = s
+        return out.view(T, H * E)
+
+    def lru_gates(self, u, recur_weight, recur_bias, input_weight, input_bias, lam, rate):
+        T, R = u.shape
+        B = recur_weight.shape[0]
+        parts = u.float().view(T, B, R // B)
+        gate = lambda w, b: torch.sigmoid(torch.einsum("tbi,boi->tbo", parts, w.float()) + b.float()).reshape(T, R)
+        r, i = gate(recur_weight, recur_bias), gate(input_weight, input_bias)
+        a = torch.exp(-rate * r * torch.nn.functional.softplus(lam.float()))
+        return a, torch.sqrt(1.0 - a * a) * i * u.float()
+
+    def lru_scan(self, a, x, state, meta, mul, mul_act, out_dtype):
+        out = torch.zeros_like(x)
+        cu, slots = meta.cu_q.tolist(), meta.state_slots.tolist()
+        for b in range(meta.num_requests):
+            h = state[slots[b]]
+            for t in range(cu[b], cu[b + 1]):
+                h = a[t] * h + x[t]
+                out[t] = h
+            state[slots[b]] = h
+        if mul is not None:
+            out = out * (mul.float() if mul_act is None else self.activation(mul.float(), mul_act))
+        return out.to(out_dtype)
+
+    def route_topk(self, x, weight, bias, top):
+        z = x.float() @ weight.float().T
+        if bias is not None:
+            z = z + bias.float()
+        order = torch.sort(z, dim=-1, descending=True, stable=True).indices[:, :top]
+        return order.to(torch.int32), torch.softmax(torch.gather(z, 1, order), -1)
+
+    def route_scale(self, hidden, experts, gates, num_experts, width):
+        T = hidden.shape[0]
+        factor = torch.zeros(T, num_experts, dtype=torch.float32, device=hidden.device)
+        factor.scatter_(1, experts.long(), gates.float())
+        routed = hidden[:, :num_experts * width].float().view(T, num_experts, width) * factor[:, :, None]
+        hidden[:, :num_experts * width] = routed.view(T, -1).to(hidden.dtype)
+        return hidden
 
     def activation(self, x, kind):
         z = x.float()
