@@ -16,6 +16,11 @@ constexpr int MAX_TAPS = 16;
 
 __device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + __expf(-x)); }
 __device__ __forceinline__ float siluf(float x) { return x / (1.f + __expf(-x)); }
+// a query temperature by position: 1 + coef * ln(floor((p + 1) / every) + 1); every < 1: none
+__device__ __forceinline__ float query_temperature(const int32_t* __restrict__ positions, int64_t t, float coef, int every) {
+  if (every < 1) return 1.f;
+  return 1.f + coef * logf(static_cast<float>((positions[t] + 1) / every) + 1.f);
+}
 // two values rounded to bfloat16 as one 32-bit word (the first in the low half)
 __device__ __forceinline__ uint32_t bf16_word(float lo, float hi) {
   return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(lo))) |
@@ -200,8 +205,8 @@ __device__ __forceinline__ float conv_at(const X* __restrict__ x, int64_t ldx, c
 template <typename X, typename W, typename O>
 __global__ void causal_conv_kernel(const X* __restrict__ x, int64_t ldx, const W* __restrict__ weight, int taps,
                                    float* __restrict__ state, O* __restrict__ out, int64_t ldo, int residual,
-                                   const int32_t* __restrict__ cu_q, const int32_t* __restrict__ token_request,
-                                   const int32_t* __restrict__ state_slots, int N) {
+                                   const float* __restrict__ bias, const int32_t* __restrict__ cu_q,
+                                   const int32_t* __restrict__ token_request, const int32_t* __restrict__ state_slots, int N) {
   const int64_t t = blockIdx.x;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= N) return;
@@ -215,6 +220,7 @@ __global__ void causal_conv_kernel(const X* __restrict__ x, int64_t ldx, const W
   float acc = conv_at(x, ldx, own, w, taps, t, i, c, N);
   const float self = to_float(x[t * ldx + c]);
   if (residual) acc += self;
+  if (bias != nullptr) acc += bias[c];
   out[t * ldo + c] = from_float<O>(acc);
   if (n == 1) {
     float keep[MAX_TAPS];
@@ -260,7 +266,8 @@ __global__ void conv_rope_kv_write_kernel(const X* __restrict__ product, int64_t
                                           C* __restrict__ v_cache, const int32_t* __restrict__ slots,
                                           const int32_t* __restrict__ cu_q, const int32_t* __restrict__ token_request,
                                           const int32_t* __restrict__ state_slots, int H, int G, int D, int E, int DP,
-                                          int block_size, int has_kv, int write) {
+                                          int block_size, int has_kv, int write, const int32_t* __restrict__ positions,
+                                          float temp_coef, int temp_every) {
   const int64_t t = blockIdx.x;
   const int head = blockIdx.y;
   const int N = H * D + (has_kv ? G * (D + E) : 0);
@@ -317,8 +324,9 @@ __global__ void conv_rope_kv_write_kernel(const X* __restrict__ product, int64_t
     }
     if (head < H) {
       Q* q = q_out + (t * H + head) * DP;
-      q[d0] = from_float<Q>(a);
-      if (d1 >= 0) q[d1] = from_float<Q>(bq);
+      const float qt = query_temperature(positions, t, temp_coef, temp_every);
+      q[d0] = from_float<Q>(a * qt);
+      if (d1 >= 0) q[d1] = from_float<Q>(bq * qt);
     } else if (write && d0 < D) {
       C* k = k_cache + ((page * G + (head - H)) * block_size + offset) * DP;
       k[d0] = from_float<C>(to_float(from_float<Q>(a)));
@@ -336,18 +344,23 @@ __global__ void sigmoid_gate_kernel(const X* __restrict__ x, int ldh, int E, con
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
     const int head = c / E, e = c % E;
     const float v = to_float(x[(t * (width / E) + head) * ldh + e]);
-    out[t * width + c] = from_float<O>(v * sigmoidf(to_float(gates[t * ldg + c])));
+    out[t * width + c] = from_float<O>(gates != nullptr ? v * sigmoidf(to_float(gates[t * ldg + c])) : v);
   }
 }
 
 // out = x / sqrt(mean(x^2) + eps) * weight * sigmoid(gate): the norm over all heads together, then the gate.
 // V channels a thread at a time (4: 16-byte loads of x, every load of a row under way before the sum).
+// A row of x may be one group of a wider row (blockIdx.y: the group, `ld` columns a row, the weight shared by the
+// groups); `silu`: the gate is g * sigmoid(g).
 template <int V, typename W, typename G, typename O>
 __global__ void rmsnorm_gate_kernel(const float* __restrict__ x, const W* __restrict__ weight, float eps,
-                                    const G* __restrict__ gates, int64_t ldg, O* __restrict__ out, int N) {
+                                    const G* __restrict__ gates, int64_t ldg, O* __restrict__ out, int N, int64_t ld,
+                                    int silu) {
   __shared__ float scratch[16];
   const int64_t t = blockIdx.x;
-  const float* row = x + t * N;
+  const float* row = x + t * ld + static_cast<int64_t>(blockIdx.y) * N;
+  if (gates != nullptr) gates += static_cast<int64_t>(blockIdx.y) * N;
+  out += t * (ld - N) + static_cast<int64_t>(blockIdx.y) * N;
   float sq = 0.f;
   for (int c = V * threadIdx.x; c < N; c += V * blockDim.x) {
     float v[V];
@@ -367,7 +380,7 @@ __global__ void rmsnorm_gate_kernel(const float* __restrict__ x, const W* __rest
       float g[V];
       loadv<V>(gates + t * ldg + c, g);
 #pragma unroll
-      for (int k = 0; k < V; ++k) v[k] *= sigmoidf(g[k]);
+      for (int k = 0; k < V; ++k) v[k] *= silu ? siluf(g[k]) : sigmoidf(g[k]);
     }
     storev<V>(out + t * N + c, v);
   }
@@ -522,8 +535,8 @@ __device__ __forceinline__ void shift_state8(float* __restrict__ own, int taps, 
 
 __global__ void causal_conv_bf16x8_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ weight,
                                           int taps, float* __restrict__ state, bf16_t* __restrict__ out, int64_t ldo,
-                                          int residual, const int32_t* __restrict__ cu_q,
-                                          const int32_t* __restrict__ token_request,
+                                          int residual, const float* __restrict__ bias,
+                                          const int32_t* __restrict__ cu_q, const int32_t* __restrict__ token_request,
                                           const int32_t* __restrict__ state_slots, int N) {
   const int64_t t = blockIdx.x;
   const int c0 = 8 * (blockIdx.y * blockDim.x + threadIdx.x);
@@ -537,6 +550,10 @@ __global__ void causal_conv_bf16x8_kernel(const bf16_t* __restrict__ x, int64_t 
   if (residual) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] += self[e];
+  }
+  if (bias != nullptr) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += bias[c0 + e];
   }
   *reinterpret_cast<uint4*>(out + t * ldo + c0) = pack_bf16x8(acc);
   if (cu_q[b + 1] - first == 1 && taps > 1) shift_state8(own, taps, c0, N, self);
@@ -556,7 +573,8 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
                                                const int32_t* __restrict__ slots, const int32_t* __restrict__ cu_q,
                                                const int32_t* __restrict__ token_request,
                                                const int32_t* __restrict__ state_slots, int T, int H, int G, int D, int E,
-                                               int DP, int block_size, int has_kv, int write) {
+                                               int DP, int block_size, int has_kv, int write,
+                                               const int32_t* __restrict__ positions, float temp_coef, int temp_every) {
   const int N = H * D + (has_kv ? G * (D + E) : 0);
   if (static_cast<int>(blockIdx.x) >= T) {
     // ---- v: 16 tokens, one channel a thread
@@ -625,6 +643,7 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
   const int64_t page = slot / block_size;
   const int offset = static_cast<int>(slot % block_size);
   const int turned = has_kv ? H + G : H;
+  const float qt = query_temperature(positions, t, temp_coef, temp_every);
   const int pair8 = pairs / 8, rest8 = (DP - 2 * pairs) / 8;
   const int per_head = pair8 + rest8;
   for (int item = threadIdx.x; item < turned * per_head; item += blockDim.x) {
@@ -648,6 +667,10 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
         a[2 * e + 1] = x0[2 * e + 1] * (cs.z * magnitude) - x1[2 * e + 1] * (cs.w * magnitude);
         c[2 * e + 1] = x1[2 * e + 1] * (cs.z * magnitude) + x0[2 * e + 1] * (cs.w * magnitude);
       }
+      if (head < H) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a[e] *= qt, c[e] *= qt;
+      }
       if (store) {
         *reinterpret_cast<uint4*>(dst + d0) = pack_bf16x8(a);
         *reinterpret_cast<uint4*>(dst + d1) = pack_bf16x8(c);
@@ -662,6 +685,10 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
       if (d0 < D) {
         conv8(product, ld, own, weight, taps, t, i, base + d0, N, a, s0);
         if (single) shift_state8(own, taps, base + d0, N, s0);
+      }
+      if (head < H) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a[e] *= qt;
       }
       if (head < H || (write && d0 < D)) *reinterpret_cast<uint4*>(dst + d0) = pack_bf16x8(a);
     }
@@ -1007,9 +1034,9 @@ extern "C" int distie_hyper_step(float* streams, int S, const float* init, const
 }
 
 extern "C" int distie_causal_conv(const void* x, int x_dtype, int64_t ldx, const void* weight, int w_dtype, int taps,
-                                  float* state, void* out, int out_dtype, int64_t ldo, int residual, const int32_t* cu_q,
-                                  const int32_t* token_request, const int32_t* state_slots, int T, int N,
-                                  hipStream_t stream) {
+                                  float* state, void* out, int out_dtype, int64_t ldo, int residual, const float* bias,
+                                  const int32_t* cu_q, const int32_t* token_request, const int32_t* state_slots, int T,
+                                  int N, hipStream_t stream) {
   if (T <= 0) return 0;
   if (taps < 1 || taps > MAX_TAPS || N < 1 || ldx < N || ldo < N || (taps > 1 && state == nullptr)) return DISTIE_BAD_ARGUMENT;
   if (x_dtype == DISTIE_BF16 && w_dtype == DISTIE_BF16 && out_dtype == DISTIE_BF16 && N % 8 == 0 && ldx % 8 == 0 &&
@@ -1018,7 +1045,7 @@ extern "C" int distie_causal_conv(const void* x, int x_dtype, int64_t ldx, const
     const int threads8 = items >= 256 ? 256 : (items >= 128 ? 128 : 64);
     causal_conv_bf16x8_kernel<<<dim3(T, (items + threads8 - 1) / threads8), threads8, 0, stream>>>(
         static_cast<const bf16_t*>(x), ldx, static_cast<const bf16_t*>(weight), taps, state, static_cast<bf16_t*>(out), ldo,
-        residual, cu_q, token_request, state_slots, N);
+        residual, bias, cu_q, token_request, state_slots, N);
     return launch_status();
   }
   const int threads = N >= 256 ? 256 : (N >= 128 ? 128 : 64);
@@ -1026,7 +1053,7 @@ extern "C" int distie_causal_conv(const void* x, int x_dtype, int64_t ldx, const
   DISTIE_DISPATCH(x_dtype, X, DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(out_dtype, O,
       causal_conv_kernel<X, W, O><<<grid, threads, 0, stream>>>(
           static_cast<const X*>(x), ldx, static_cast<const W*>(weight), taps, state, static_cast<O*>(out), ldo, residual,
-          cu_q, token_request, state_slots, N))));
+          bias, cu_q, token_request, state_slots, N))));
   return launch_status();
 }
 
@@ -1046,8 +1073,10 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
                                          void* q_out, void* k_cache, void* v_cache, int cache_dtype, const int32_t* slots,
                                          const int32_t* cu_q, const int32_t* token_request, const int32_t* state_slots,
                                          int T, int H, int G, int D, int E, int DP, int block_size, int has_kv, int write,
-                                         hipStream_t stream) {
+                                         const int32_t* positions, float temp_coef, int temp_every, hipStream_t stream) {
+  // temp_every >= 1: q of the token at position p times 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)
   if (T <= 0) return 0;
+  if (temp_every >= 1 && positions == nullptr) return DISTIE_BAD_ARGUMENT;
   if (H < 1 || G < 1 || D < 1 || E < 1 || DP < D || DP < E || block_size < 1 || pairs < 0 || 2 * pairs > D ||
       taps < 0 || taps > MAX_TAPS)
     return DISTIE_BAD_ARGUMENT;
@@ -1063,7 +1092,8 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
     conv_rope_kv_write_bf16_kernel<<<T + v_blocks, threads8, 0, stream>>>(
         static_cast<const bf16_t*>(product), ld, static_cast<const bf16_t*>(weight), taps, state,
         static_cast<const float2*>(table), pairs, magnitude, static_cast<bf16_t*>(q_out), static_cast<bf16_t*>(k_cache),
-        static_cast<bf16_t*>(v_cache), slots, cu_q, token_request, state_slots, T, H, G, D, E, DP, block_size, has_kv, write);
+        static_cast<bf16_t*>(v_cache), slots, cu_q, token_request, state_slots, T, H, G, D, E, DP, block_size, has_kv, write,
+        positions, temp_coef, temp_every);
     return launch_status();
   }
   const int work = DP - pairs > E ? DP - pairs : E;
@@ -1074,15 +1104,16 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
       conv_rope_kv_write_kernel<X, W, X, C><<<grid, threads, 0, stream>>>(
           static_cast<const X*>(product), ld, static_cast<const W*>(weight), taps, state, static_cast<const float2*>(table),
           pairs, magnitude, static_cast<X*>(q_out), static_cast<C*>(k_cache), static_cast<C*>(v_cache), slots, cu_q,
-          token_request, state_slots, H, G, D, E, DP, block_size, has_kv, write))));
+          token_request, state_slots, H, G, D, E, DP, block_size, has_kv, write, positions, temp_coef, temp_every))));
   return launch_status();
 }
 
 extern "C" int distie_sigmoid_gate(const void* x, int x_dtype, int ldh, int E, const void* gates, int g_dtype, int64_t ldg,
                                    void* out, int out_dtype, int T, int width, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (E < 1 || width < 1 || width % E || ldh < E || ldg < width) return DISTIE_BAD_ARGUMENT;
-  if (x_dtype == DISTIE_BF16 && g_dtype == DISTIE_BF16 && out_dtype == DISTIE_BF16 && E % 8 == 0 && ldh % 8 == 0 &&
+  if (E < 1 || width < 1 || width % E || ldh < E || (gates != nullptr && ldg < width)) return DISTIE_BAD_ARGUMENT;
+  if (gates == nullptr) g_dtype = x_dtype;
+  if (gates != nullptr && x_dtype == DISTIE_BF16 && g_dtype == DISTIE_BF16 && out_dtype == DISTIE_BF16 && E % 8 == 0 && ldh % 8 == 0 &&
       ldg % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(gates) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
     const int64_t pieces = static_cast<int64_t>(T) * (width / 8);
     const int blocks8 = static_cast<int>(pieces / 256 + 1 < 16384 ? pieces / 256 + 1 : 16384);
@@ -1100,19 +1131,23 @@ extern "C" int distie_sigmoid_gate(const void* x, int x_dtype, int ldh, int E, c
 }
 
 extern "C" int distie_rmsnorm_gate(const float* x, const void* weight, int w_dtype, float eps, const void* gates,
-                                   int g_dtype, int64_t ldg, void* out, int out_dtype, int T, int N, hipStream_t stream) {
+                                   int g_dtype, int64_t ldg, void* out, int out_dtype, int T, int N, int groups, int silu,
+                                   hipStream_t stream) {
+  // N: columns of one norm; a row of x, of the gates and of out holds `groups` of them side by side
   if (T <= 0) return 0;
-  if (N < 1 || (gates != nullptr && ldg < N)) return DISTIE_BAD_ARGUMENT;
+  if (N < 1 || groups < 1 || (gates != nullptr && ldg < static_cast<int64_t>(N) * groups)) return DISTIE_BAD_ARGUMENT;
   if (gates == nullptr) g_dtype = DISTIE_F32;
   const bool wide = N % 8 == 0 && ldg % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
                     reinterpret_cast<uintptr_t>(weight) % 16 == 0 && reinterpret_cast<uintptr_t>(gates) % 16 == 0 &&
                     reinterpret_cast<uintptr_t>(out) % 16 == 0;
   const int per = wide ? N / 4 : N;
   const int threads = per >= 1024 ? 1024 : (per >= 512 ? 512 : (per >= 256 ? 256 : (per >= 128 ? 128 : 64)));
+  const dim3 grid(T, groups);
+  const int64_t ld = static_cast<int64_t>(N) * groups;
 #define DISTIE_NORM_GATE(V)                                                                                  \
   DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(g_dtype, G, DISTIE_DISPATCH(out_dtype, O,                      \
-      rmsnorm_gate_kernel<V, W, G, O><<<T, threads, 0, stream>>>(                                            \
-          x, static_cast<const W*>(weight), eps, static_cast<const G*>(gates), ldg, static_cast<O*>(out), N))))
+      rmsnorm_gate_kernel<V, W, G, O><<<grid, threads, 0, stream>>>(                                         \
+          x, static_cast<const W*>(weight), eps, static_cast<const G*>(gates), ldg, static_cast<O*>(out), N, ld, silu))))
   if (wide) {
     DISTIE_NORM_GATE(4);
   } else {

@@ -127,6 +127,18 @@ class PendingProduct(_NotATensorYet):
         self.device = x.device
 
 
+class NormedSum(_NotATensorYet):
+    """scale * sum_i rmsnorm(terms[i]) * weights[i], not computed yet: if what happens to it next is the norm behind
+    its sub-layer and the sum into the residual stream, one kernel does all of it (`distie_norm_chain`); anything else
+    sees the finished float32 tensor through `HipOps.dense`."""
+
+    def __init__(self, terms, weights, eps: float, scale: float) -> None:
+        self.terms, self.weights, self.eps, self.scale = terms, weights, eps, scale
+        self.dtype = torch.float32
+        self.shape = terms[0].shape
+        self.device = terms[0].device
+
+
 class HipOps(Ops):
     # Steps of up to FUSED_MAX_ROWS rows can run their products with the norm in front and the residual sum behind
     # folded in (six launches a layer instead of eight, no partial sums handed on). On the device that is no
@@ -293,12 +305,19 @@ class HipOps(Ops):
         o.distie_decode_norm_product.argtypes = [_P, _P, _F, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P,
                                                  _I, _I, _I, _I, _I, _P]
         o.distie_hyper_step.argtypes = [_P, _I, _P, _P, _I, _I, _P, _I, _L, _I, _P, _P, _P, _P, _I, _I, _F, _P, _I, _I, _I, _P]
-        o.distie_causal_conv.argtypes = [_P, _I, _L, _P, _I, _I, _P, _P, _I, _L, _I, _P, _P, _P, _I, _I, _P]
+        o.distie_causal_conv.argtypes = [_P, _I, _L, _P, _I, _I, _P, _P, _I, _L, _I, _P, _P, _P, _P, _I, _I, _P]
         o.distie_conv_state.argtypes = [_P, _I, _L, _I, _P, _P, _P, _I, _I, _I, _P]
         o.distie_conv_rope_kv_write.argtypes = [_P, _I, _L, _P, _I, _I, _P, _P, _I, _F, _P, _P, _P, _I, _P, _P, _P, _P,
-                                                _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]
+                                                _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P]
         o.distie_sigmoid_gate.argtypes = [_P, _I, _I, _I, _P, _I, _L, _P, _I, _I, _I, _P]
-        o.distie_rmsnorm_gate.argtypes = [_P, _P, _I, _F, _P, _I, _L, _P, _I, _I, _I, _P]
+        o.distie_rmsnorm_gate.argtypes = [_P, _P, _I, _F, _P, _I, _L, _P, _I, _I, _I, _I, _I, _P]
+        o.distie_norm_chain.argtypes = [_P, _I, _I, _P, _P, _I, _I, _P, _F, _F, _P, _F, _P, _P, _F, _P, _I, _P, _I, _I, _P]
+        o.distie_gated_decay_scan.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _P]
+        o.distie_lru_gates.argtypes = [_P, _I, _L, _P, _P, _P, _P, _I, _P, _F, _P, _P, _I, _I, _I, _P]
+        o.distie_lru_scan.argtypes = [_P, _P, _P, _P, _I, _L, _I, _P, _I, _P, _P, _I, _I, _P]
+        o.distie_route_topk.argtypes = [_P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _P]
+        o.distie_route_scale.argtypes = [_P, _I, _L, _P, _P, _I, _I, _I, _I, _P]
+        o.distie_scale_f32.argtypes = [_P, _L, _F, _P]
         o.distie_activation.argtypes = [_P, _I, _I, _P, _I, _L, _I, _P]
         o.distie_decay_scan.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]
         o.distie_decay_scan_chunked.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
@@ -445,6 +464,8 @@ class HipOps(Ops):
             return self._rmsnorm_now(x.residual, x.weight, x.eps, x.dtype)
         if isinstance(x, PendingProduct):
             return self._linear(x.x, x.weight, x.bias, x.dtype, lazy=False)
+        if isinstance(x, NormedSum):
+            return self._norm_chain(x.terms, x.weights, x.eps, x.scale, None, None, None, None)
         if not isinstance(x, PartialSums):
             return x
         out = torch.empty(tuple(x.shape), dtype=x.dtype, device=self.device)
@@ -834,8 +855,11 @@ class HipOps(Ops):
         """May return `PartialSums` (see there)."""
         return self._linear(x, weight, bias, x.dtype, partial_ok=True, lazy=True)
 
-    def linear_f32out(self, x, weight):
-        return self._linear(x, weight, None, torch.float32)
+    def linear_f32out(self, x, weight, bias=None, scale=1.0):
+        out = self._linear(x, weight, bias, torch.float32)
+        if scale != 1.0:
+            _check(self._ops.distie_scale_f32(out.data_ptr(), out.numel(), float(scale), self._stream()), "scale_f32")
+        return out
 
     def rope_kv_write(self, qkv, meta: BatchMeta, group, k_cache, v_cache, inv_freq, num_heads, num_kv_heads,
                       head_dim, write):
@@ -1078,23 +1102,27 @@ class HipOps(Ops):
         _mark_written(streams)
         return streams, h
 
-    def causal_conv(self, x, weight, state, meta, residual=False):
+    def causal_conv(self, x, weight, state, meta, residual=False, bias=None):
         x = self.dense(x)
-        self._own(x, weight, state)
+        self._own(weight, state, bias)
         T, N = x.shape
+        x_ptr, ldx = self._rows_view(x, N)
         taps = weight.shape[1]
         if tuple(weight.shape) != (N, taps) or T != meta.num_tokens:
             raise KernelError("causal_conv: weight must be [channels of x, taps], x the step's rows")
+        if bias is not None and (bias.dtype != torch.float32 or tuple(bias.shape) != (N,)):
+            raise KernelError("causal_conv: bias must be float32 [channels]")
         self._check_conv_state(state, taps, N)
-        out = torch.empty_like(x)
+        out = torch.empty((T, N), dtype=x.dtype, device=self.device)
         _check(self._ops.distie_causal_conv(
-            x.data_ptr(), _code(x), N, weight.data_ptr(), _code(weight), taps, state.data_ptr() if taps > 1 else None,
-            out.data_ptr(), _code(out), N, 1 if residual else 0, meta.cu_q.data_ptr(), meta.token_request.data_ptr(),
-            meta.state_slots.data_ptr(), T, N, self._stream()), "causal_conv")
+            x_ptr, _code(x), ldx, weight.data_ptr(), _code(weight), taps, state.data_ptr() if taps > 1 else None,
+            out.data_ptr(), _code(out), N, 1 if residual else 0, bias.data_ptr() if bias is not None else None,
+            meta.cu_q.data_ptr(), meta.token_request.data_ptr(), meta.state_slots.data_ptr(), T, N, self._stream()),
+            "causal_conv")
         if taps > 1 and not meta.all_decode:
             # requests that bring one row moved their state on in the kernel above; the others here, once all
             # rows of the step have read the old one
-            _check(self._ops.distie_conv_state(x.data_ptr(), _code(x), N, taps, state.data_ptr(), meta.cu_q.data_ptr(),
+            _check(self._ops.distie_conv_state(x_ptr, _code(x), ldx, taps, state.data_ptr(), meta.cu_q.data_ptr(),
                                                meta.state_slots.data_ptr(), meta.num_requests, N, 1, self._stream()),
                    "conv_state")
         if taps > 1:
@@ -1107,7 +1135,7 @@ class HipOps(Ops):
                               f"[slots, {taps - 1}, {channels}]")
 
     def conv_rope_kv_write(self, product, conv_weight, state, meta, group, k_cache, v_cache, inv_freq, magnitude,
-                           num_heads, num_kv_heads, dim, value_dim, padded_dim, has_kv, write):
+                           num_heads, num_kv_heads, dim, value_dim, padded_dim, has_kv, write, q_temp=None):
         product = self.dense(product)
         self._own(product, conv_weight, state, k_cache, v_cache, inv_freq)
         T, W = product.shape
@@ -1133,7 +1161,8 @@ class HipOps(Ops):
             ptr(k_cache) if write else None, ptr(v_cache) if write else None, _code(k_cache) if write else _code(product),
             meta.groups[group].slots.data_ptr() if write else None, meta.cu_q.data_ptr(), meta.token_request.data_ptr(),
             meta.state_slots.data_ptr(), T, num_heads, num_kv_heads, dim, value_dim, padded_dim, meta.block_size,
-            1 if has_kv else 0, 1 if write else 0, self._stream()), "conv_rope_kv_write")
+            1 if has_kv else 0, 1 if write else 0, meta.positions.data_ptr(), float(q_temp[0]) if q_temp else 0.0,
+            int(q_temp[1]) if q_temp else 0, self._stream()), "conv_rope_kv_write")
         if taps > 1:
             if not meta.all_decode:
                 # (requests that bring one row had their state moved on by the kernel above)
@@ -1149,9 +1178,10 @@ class HipOps(Ops):
         T = x.shape[0]
         if x.shape[1] != num_heads * head_stride or width > head_stride:
             raise KernelError("sigmoid_gate: x must be [T, heads * head_stride]")
-        g_ptr, g_ld = self._rows_view(gates, num_heads * width)
+        g_ptr, g_ld = self._rows_view(gates, num_heads * width) if gates is not None else (None, 0)
         out = torch.empty((T, num_heads * width), dtype=x.dtype, device=self.device)
-        _check(self._ops.distie_sigmoid_gate(x.data_ptr(), _code(x), head_stride, width, g_ptr, _code(gates), g_ld,
+        _check(self._ops.distie_sigmoid_gate(x.data_ptr(), _code(x), head_stride, width, g_ptr,
+                                             _code(gates) if gates is not None else _code(x), g_ld,
                                              out.data_ptr(), _code(out), T, num_heads * width, self._stream()),
                "sigmoid_gate")
         return out
@@ -1198,19 +1228,182 @@ class HipOps(Ops):
         _mark_written(state)
         return out
 
-    def rmsnorm_gate(self, x, weight, eps, gates, out_dtype):
+    def rmsnorm_gate(self, x, weight, eps, gates, out_dtype, group=None, gate="sigmoid"):
         self._own(x, weight)
-        if x.dtype != torch.float32 or x.dim() != 2 or tuple(weight.shape) != (x.shape[1],):
-            raise KernelError("rmsnorm_gate: x must be float32 [T, N], weight [N]")
+        if gate not in ("sigmoid", "silu"):
+            raise KernelError(f"rmsnorm_gate: no gate named {gate!r}")
+        if x.dtype != torch.float32 or x.dim() != 2 or (group is not None and (group < 1 or x.shape[1] % group)) or \
+                tuple(weight.shape) != (group or x.shape[1],):
+            raise KernelError("rmsnorm_gate: x must be float32 [T, N], weight [N] (or [group], N a multiple of it)")
         T, N = x.shape
         g_ptr, g_ld, g_code = None, 0, _F32
         if gates is not None:
             g_ptr, g_ld = self._rows_view(gates, N)
             g_code = _code(gates)
         out = torch.empty((T, N), dtype=out_dtype, device=self.device)
+        size = group or N
         _check(self._ops.distie_rmsnorm_gate(x.data_ptr(), weight.data_ptr(), _code(weight), float(eps), g_ptr, g_code,
-                                             g_ld, out.data_ptr(), _code(out), T, N, self._stream()), "rmsnorm_gate")
+                                             g_ld, out.data_ptr(), _code(out), T, size, N // size,
+                                             1 if gate == "silu" else 0, self._stream()), "rmsnorm_gate")
         return out
+
+    # ---- norms behind sub-layers, mixers side by side, gated states, routers (csrc/recurrent.hip)
+    def _term(self, value):
+        """(tensor, slices) of a sub-layer's result as the norm kernels read it."""
+        if isinstance(value, NormedSum):
+            value = self.dense(value)
+        if isinstance(value, (PendingNorm, PendingProduct)):
+            value = self.dense(value)
+        if isinstance(value, PartialSums):
+            self._own(value.data)
+            return value.data, value.slices
+        self._own(value)
+        return value, 1
+
+    def _norm_chain(self, terms, weights, term_eps, scale, post, residual, pre, out_dtype):
+        held = [self._term(t) for t in terms]
+        T, C = held[0][0].shape[-2:]
+        for tensor, _ in held:
+            if tuple(tensor.shape[-2:]) != (T, C):
+                raise KernelError("norm chain: the terms must all be [T, C]")
+        vectors = list(weights or []) + [v[0] for v in (post, pre) if v is not None]
+        self._own(*vectors)
+        for w in vectors:
+            if w.dtype != torch.float32 or tuple(w.shape) != (C,):
+                raise KernelError("norm chain: norm weights are float32 [C]")
+        if residual is not None:
+            self._own(residual)
+            if residual.dtype != torch.float32 or tuple(residual.shape) != (T, C):
+                raise KernelError("norm chain: the residual is float32 [T, C]")
+        out = y = None
+        if residual is None:
+            y = torch.empty((T, C), dtype=torch.float32, device=self.device)
+        elif pre is not None:
+            out = torch.empty((T, C), dtype=out_dtype, device=self.device)
+        (t0, s0), (t1, s1) = held[0], (held[1] if len(held) > 1 else (None, 1))
+        ptr = lambda t: t.data_ptr() if t is not None else None
+        _check(self._ops.distie_norm_chain(
+            t0.data_ptr(), _code(t0), s0, ptr(weights[0]) if weights else None, ptr(t1), _code(t1) if t1 is not None else _F32,
+            s1, ptr(weights[1]) if weights and len(weights) > 1 else None, float(term_eps), float(scale),
+            ptr(post[0]) if post else None, float(post[1]) if post else 0.0, ptr(residual),
+            ptr(pre[0]) if pre else None, float(pre[1]) if pre else 0.0, ptr(out), _code(out) if out is not None else _F32,
+            ptr(y), T, C, self._stream()), "norm_chain")
+        if residual is not None:
+            _mark_written(residual)
+        return out if residual is not None else y
+
+    def normed_sum(self, terms, weights, eps, scale):
+        if not 1 <= len(terms) <= 2 or len(weights) != len(terms):
+            raise KernelError("normed_sum takes one or two terms, a weight for each")
+        return NormedSum(list(terms), [self._f32(w) for w in weights], float(eps), float(scale))
+
+    @staticmethod
+    def _f32(weight):
+        """A norm's weight as float32 (a bfloat16 value is one exactly); kept on the tensor."""
+        if weight.dtype == torch.float32:
+            return weight
+        held = getattr(weight, "_distie_f32", None)
+        if held is None:
+            held = weight._distie_f32 = weight.float()
+        return held
+
+    def add_normed(self, residual, delta, weight, eps):
+        self.add_normed_rmsnorm(residual, delta, weight, eps, None, 0.0, None)
+
+    def add_normed_rmsnorm(self, residual, delta, post_weight, post_eps, weight, eps, out_dtype):
+        post = (self._f32(post_weight), post_eps)
+        pre = (self._f32(weight), eps) if weight is not None else None
+        if isinstance(delta, NormedSum):
+            return self._norm_chain(delta.terms, delta.weights, delta.eps, delta.scale, post, residual, pre, out_dtype)
+        return self._norm_chain([delta], None, 0.0, 1.0, post, residual, pre, out_dtype)
+
+    def gated_decay_scan(self, product, decay_logits, state, meta, num_heads, dim, value_dim, q_scale, tau):
+        product = self.dense(product)
+        self._own(product, decay_logits, state)
+        T, W = product.shape
+        if T != meta.num_tokens or W < num_heads * (2 * dim + value_dim):
+            raise KernelError("gated_decay_scan: the product does not match the batch or the head counts")
+        if decay_logits.dtype != torch.float32 or tuple(decay_logits.shape) != (T, num_heads * dim):
+            raise KernelError("gated_decay_scan: the decay's logits are float32 [T, heads * dim]")
+        if state.dtype != torch.float32 or tuple(state.shape[1:]) != (num_heads, dim, value_dim):
+            raise KernelError("gated_decay_scan: the state is float32 [slots, heads, dim, value_dim]")
+        out = torch.empty((T, num_heads * value_dim), dtype=torch.float32, device=self.device)
+        _check(self._ops.distie_gated_decay_scan(
+            product.data_ptr(), _code(product), W, decay_logits.data_ptr(), state.data_ptr(), out.data_ptr(),
+            meta.cu_q.data_ptr(), meta.state_slots.data_ptr(), meta.num_requests, num_heads, dim, value_dim,
+            float(q_scale), float(tau), self._stream()), "gated_decay_scan")
+        _mark_written(state)
+        return out
+
+    def lru_gates(self, u, recur_weight, recur_bias, input_weight, input_bias, lam, rate):
+        u = self.dense(u)
+        self._own(recur_weight, recur_bias, input_weight, input_bias, lam)
+        T, R = u.shape
+        u_ptr, ldu = self._rows_view(u, R)
+        blocks = recur_weight.shape[0]
+        n = R // max(blocks, 1)
+        if recur_weight.dim() != 3 or tuple(recur_weight.shape) != (blocks, n, n) or blocks * n != R or \
+                input_weight.shape != recur_weight.shape or input_weight.dtype != recur_weight.dtype:
+            raise KernelError("lru_gates: the gates' weights are [blocks, R / blocks, R / blocks], of one dtype")
+        for t in (recur_bias, input_bias, lam):
+            if t.dtype != torch.float32 or t.numel() != R:
+                raise KernelError("lru_gates: biases and lam are float32 with R elements")
+        a = torch.empty((T, R), dtype=torch.float32, device=self.device)
+        x = torch.empty((T, R), dtype=torch.float32, device=self.device)
+        _check(self._ops.distie_lru_gates(u_ptr, _code(u), ldu, recur_weight.data_ptr(), recur_bias.data_ptr(),
+                                          input_weight.data_ptr(), input_bias.data_ptr(), _code(recur_weight),
+                                          lam.data_ptr(), float(rate), a.data_ptr(), x.data_ptr(), T, R, blocks,
+                                          self._stream()), "lru_gates")
+        return a, x
+
+    def lru_scan(self, a, x, state, meta, mul, mul_act, out_dtype):
+        self._own(a, x, state)
+        T, R = a.shape
+        if a.dtype != torch.float32 or x.dtype != torch.float32 or x.shape != a.shape or T != meta.num_tokens:
+            raise KernelError("lru_scan: a and x are float32 [T, R], the step's rows")
+        if state.dtype != torch.float32 or tuple(state.shape[1:]) != (R,):
+            raise KernelError("lru_scan: the state is float32 [slots, R]")
+        kind = -1
+        if mul_act is not None:
+            if mul_act not in self.ACTIVATIONS:
+                raise KernelError(f"no activation named {mul_act!r}")
+            kind = self.ACTIVATIONS[mul_act]
+        m_ptr, m_ld, m_code = None, 0, _F32
+        if mul is not None:
+            m_ptr, m_ld = self._rows_view(mul, R)
+            m_code = _code(mul)
+        out = torch.empty((T, R), dtype=out_dtype, device=self.device)
+        _check(self._ops.distie_lru_scan(a.data_ptr(), x.data_ptr(), state.data_ptr(), m_ptr, m_code, m_ld, kind,
+                                         out.data_ptr(), _code(out), meta.cu_q.data_ptr(), meta.state_slots.data_ptr(),
+                                         meta.num_requests, R, self._stream()), "lru_scan")
+        _mark_written(state)
+        return out
+
+    def route_topk(self, x, weight, bias, top):
+        x = self.dense(x)
+        self._own(x, weight, bias)
+        T, C = x.shape
+        E = weight.shape[0]
+        if tuple(weight.shape) != (E, C) or (bias is not None and (bias.dtype != torch.float32 or tuple(bias.shape) != (E,))):
+            raise KernelError("route_topk: weight [experts, C], bias float32 [experts]")
+        experts = torch.empty((T, top), dtype=torch.int32, device=self.device)
+        gates = torch.empty((T, top), dtype=torch.float32, device=self.device)
+        _check(self._ops.distie_route_topk(x.data_ptr(), _code(x), weight.data_ptr(), _code(weight),
+                                           bias.data_ptr() if bias is not None else None, experts.data_ptr(),
+                                           gates.data_ptr(), T, C, E, int(top), self._stream()), "route_topk")
+        return experts, gates
+
+    def route_scale(self, hidden, experts, gates, num_experts, width):
+        hidden = self.dense(hidden)
+        self._own(hidden, experts, gates)
+        T, top = experts.shape
+        if experts.dtype != torch.int32 or gates.dtype != torch.float32 or gates.shape != experts.shape or \
+                hidden.shape[0] != T or hidden.shape[1] < num_experts * width:
+            raise KernelError("route_scale: experts int32 and gates float32 [T, top], hidden [T, >= experts * width]")
+        _check(self._ops.distie_route_scale(hidden.data_ptr(), _code(hidden), hidden.shape[1], experts.data_ptr(),
+                                            gates.data_ptr(), T, top, num_experts, width, self._stream()), "route_scale")
+        _mark_written(hidden)
+        return hidden
 
     def activation(self, x, kind):
         if kind not in self.ACTIVATIONS:
