@@ -17,7 +17,7 @@ serves it), points at batch 1 and 32, and a cache that takes the card's memory u
 the time to the first token and the time per output token after it, defined as the reference's load
 generator defines them (benchmarks/load/stats.py:29-34, 67-86).
 
-`--design musutar [--size w1024|w2048|w4096]`: prefill and decode of the Musutar decoder beside a Qwen2 decoder of
+`--design musutar|duparax [--size w1024|w2048|w4096]`: prefill and decode of that decoder beside a Qwen2 decoder of
 equal width, depth, heads and weights, at layer sizes of real models; one JSON line with both for every size.
 
 Random weights N(0, 0.02), seeded uniform token ids.
@@ -236,6 +236,59 @@ def qwen2_equal(size):
                 rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=8192)
 
 
+def duparax_config(size):
+    """Groups of four layers: mixers side by side (softmax attention with keys of half the head size beside gated linear
+    attention), a recurrent layer, and two more of the first kind; dense feed-forwards alternate with mixtures of eight
+    experts of a quarter of the dense size, two a token, beside a shared one."""
+    z = DESIGN_SIZES[size]
+    layers = []
+    for i in range(z["layers"]):
+        if i % 2 == 0:
+            mlp = {"kind": "dense", "ff": z["ff"]}
+        else:
+            mlp = {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": z["ff"] // 4},
+                   "shared": {"ff": z["ff"] // 4}}
+        if i % 4 == 1:
+            layers.append({"type": "rglru", "mlp": mlp,
+                           "mixer": {"width": z["width"], "blocks": z["width"] // 128, "conv": 4}})
+            continue
+        left = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"] // 2, "vdim": z["dim"],
+                "scale": (z["dim"] // 2) ** -0.5, "q_temp": {"coef": 0.5, "every": 64}}
+        right = {"heads": z["heads"] // 2, "dim": z["dim"] // 2, "vdim": z["dim"], "tau": 16.0, "rank": 32}
+        layers.append({"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp})
+    return {"architecture": "Duparax", "vocab": DESIGN_VOCAB, "width": z["width"], "norm": {"eps": 1e-6},
+            "logit_scale": 0.5, "layers": layers}
+
+
+def qwen2_of_weights(size, layer_weights):
+    """The Qwen2 decoder with the same width, depth and heads and a feed-forward sized so that its layers hold as many
+    weights as the other design's layers do on average."""
+    z = DESIGN_SIZES[size]
+    C, q, kv = z["width"], z["heads"] * z["dim"], z["kv_heads"] * z["dim"]
+    inter = int(layer_weights - C * (q + 2 * kv) - q * C) // (3 * C) // 32 * 32
+    return dict(COMMON, num_hidden_layers=z["layers"], hidden_size=C, num_attention_heads=z["heads"],
+                num_key_value_heads=z["kv_heads"], head_dim=z["dim"], intermediate_size=inter, vocab_size=DESIGN_VOCAB,
+                rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=8192)
+
+
+def design_pair(design, size):
+    """(the design's configuration, the Qwen2 configuration of equal size)"""
+    if design == "musutar":
+        return musutar_config(size), qwen2_equal(size)
+    from distie_amd.config import config_from_dict
+    from distie_amd.engine.model import Model
+
+    config = duparax_config(size)
+    total = 0
+    for name, spec in Model.declare(config_from_dict(config).model_spec()).items():
+        if name.startswith("l"):
+            count = 1
+            for n in spec.shape:
+                count *= int(n)
+            total += count
+    return config, qwen2_of_weights(size, total / len(config["layers"]))
+
+
 def design_run(args) -> int:
     import torch
 
@@ -247,7 +300,7 @@ def design_run(args) -> int:
     sizes = {}
     for size in ([args.size] if args.size else list(DESIGN_SIZES)):
         row = {}
-        for name, config in (("musutar", musutar_config(size)), ("qwen2", qwen2_equal(size))):
+        for name, config in zip((args.design, "qwen2"), design_pair(args.design, size)):
             llm = LLM(config=config, random_weights=True, seed=0, dtype=args.dtype, block_size=BLOCK_SIZE,
                       num_blocks=pages, max_seqs=args.batch, token_budget=TOKEN_BUDGET, use_graphs=True,
                       max_model_len=max(8192, tokens_per_request), tune_products=not args.no_tune)
@@ -266,7 +319,7 @@ def design_run(args) -> int:
             del llm
             torch.cuda.empty_cache()
         sizes[size] = dict(DESIGN_SIZES[size], **row)
-    print(json.dumps({"metric": "prefill and decode tok/s, Musutar beside Qwen2 at equal size", "unit": "tok/s",
+    print(json.dumps({"metric": f"prefill and decode tok/s, {args.design.capitalize()} beside Qwen2 at equal size", "unit": "tok/s",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype, "data": "synthetic",
                       "config": {"batch": args.batch, "context": context, "prefill_tokens": prefill_tokens,
                                  "vocab": DESIGN_VOCAB, "block_size": BLOCK_SIZE, "captured_decode": True},
@@ -297,7 +350,7 @@ def main() -> int:
                         help="size the cache from free memory (the default for --shape 32b and --serve: 0.9)")
     parser.add_argument("--packed-weights", default=None, metavar="ROLES",
                         help="packed copies only for these products (qkv,attn_out,gate_up,down,head); 'none' for no copies")
-    parser.add_argument("--design", default=None, choices=["musutar"],
+    parser.add_argument("--design", default=None, choices=["musutar", "duparax"],
                         help="instead of the workload above: this design beside a Qwen2 decoder of equal size, prefill and decode")
     parser.add_argument("--size", default=None, choices=sorted(DESIGN_SIZES), help="with --design: one size instead of all")
     args = parser.parse_args()

@@ -162,6 +162,226 @@ gated_decay_scan_kernel(const X* __restrict__ product, int64_t ld, const float* 
 }
 
 // ---------------------------------------------------------------------------------------------------
+// The same recurrence over portions of prompts, in chunks of 64 rows that run side by side. With L the rows of a
+// chunk, S the state in front of it and c_i[d] = sum_{m <= i} ln alpha_m[d] (the chunk's own running sum, <= 0):
+//   sums:     P[d][e] = sum_j exp(c_L[d] - c_j[d]) k_j[d] v_j[e],   G[d] = exp(c_L[d])           (each chunk alone)
+//   states:   S_next = diag(G) S + P, chunk after chunk; S (the state in front) takes P's place in the scratch
+//   outputs:  o_i[e] = sum_d q_i[d] exp(c_i[d]) S[d][e] + sum_{j <= i} (sum_d q_i[d] k_j[d] exp(c_i[d] - c_j[d])) v_j[e]
+// Every exponent is <= 0: nothing grows, however fast a channel forgets, and no quotient of decays is ever formed
+// (the decay differs from channel to channel, so the scores of a pair of rows are summed channel by channel with the
+// pair's own factor). Float32 throughout, FMAs on tiles held in LDS; a chunk's table entry is {request, first row,
+// rows, unused}.
+constexpr int GS_L = 64;
+constexpr int GS_PAD = 68;        // row stride of the transposed tiles: keeps 16-byte reads aligned
+
+// ln alpha of the chunk's rows into `c` (laid out [d][GS_PAD], rows beyond the chunk 0), then the running sums down
+// the rows, one thread a channel
+__device__ __forceinline__ void decay_prefix(float* __restrict__ c, const float* __restrict__ logits, int64_t row0, int len,
+                                             int head, int H, int D, float tau) {
+  for (int idx = threadIdx.x; idx < GS_L * D; idx += blockDim.x) {
+    const int j = idx / D, d = idx % D;
+    c[d * GS_PAD + j] = j < len ? log_sigmoid(logits[((row0 + j) * H + head) * D + d]) / tau : 0.f;
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float run = 0.f;
+    for (int j = 0; j < GS_L; ++j) {
+      run += c[d * GS_PAD + j];
+      c[d * GS_PAD + j] = run;
+    }
+  }
+  __syncthreads();
+}
+
+template <typename X>
+__global__ void __launch_bounds__(256)
+gated_chunk_sums_kernel(const X* __restrict__ product, int64_t ld, const float* __restrict__ logits, float tau,
+                        float* __restrict__ scratch, float* __restrict__ totals, const int4* __restrict__ chunks, int H,
+                        int D, int E) {
+  extern __shared__ float lds[];
+  float* Ct = lds;                        // [D][68]
+  float* Ks = Ct + D * GS_PAD;            // [64][D]: k_j[d] exp(c_L[d] - c_j[d])
+  float* Vs = Ks + GS_L * D;              // [64][64]
+  const int c = blockIdx.x, head = blockIdx.y, e0 = blockIdx.z * 64;
+  const int4 chunk = chunks[c];
+  const int64_t row0 = chunk.y;
+  const int len = chunk.z;
+  decay_prefix(Ct, logits, row0, len, head, H, D, tau);
+  for (int idx = threadIdx.x; idx < GS_L * D; idx += blockDim.x) {
+    const int j = idx / D, d = idx % D;
+    const float k = j < len ? to_float(product[(row0 + j) * ld + (H + head) * D + d]) : 0.f;
+    Ks[j * D + d] = k * expf(Ct[d * GS_PAD + GS_L - 1] - Ct[d * GS_PAD + j]);
+  }
+  for (int idx = threadIdx.x; idx < GS_L * 64; idx += blockDim.x) {
+    const int j = idx / 64, col = idx % 64;
+    Vs[idx] = (j < len && e0 + col < E) ? to_float(product[(row0 + j) * ld + 2 * H * D + head * E + e0 + col]) : 0.f;
+  }
+  if (blockIdx.z == 0)
+    for (int d = threadIdx.x; d < D; d += blockDim.x)
+      totals[(static_cast<int64_t>(c) * H + head) * D + d] = expf(Ct[d * GS_PAD + GS_L - 1]);
+  __syncthreads();
+  const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+  float acc[2][4][4] = {};
+#pragma unroll 4
+  for (int j = 0; j < len; ++j) {
+    const float4 v4 = *reinterpret_cast<const float4*>(Vs + j * 64 + 4 * tx);
+    const float v[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int d0 = 4 * ty + 64 * s;
+      if (d0 >= D) break;
+      const float4 k4 = *reinterpret_cast<const float4*>(Ks + j * D + d0);
+      const float k[4] = {k4.x, k4.y, k4.z, k4.w};
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[s][a][b] += k[a] * v[b];
+    }
+  }
+  float* dst = scratch + (static_cast<int64_t>(c) * H + head) * D * E;
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int d = 4 * ty + 64 * s + a;
+      if (d >= D) continue;
+      const int e = e0 + 4 * tx;                          // E is a multiple of 4: four columns are there or none
+      if (e < E)
+        *reinterpret_cast<float4*>(dst + static_cast<int64_t>(d) * E + e) =
+            float4{acc[s][a][0], acc[s][a][1], acc[s][a][2], acc[s][a][3]};
+    }
+}
+
+__global__ void gated_chunk_states_kernel(float* __restrict__ scratch, const float* __restrict__ totals,
+                                          float* __restrict__ state, const int32_t* __restrict__ request_chunks,
+                                          const int32_t* __restrict__ state_slots, int H, int D, int E) {
+  const int b = blockIdx.x, head = blockIdx.y;
+  const int idx = blockIdx.z * blockDim.x + threadIdx.x;
+  if (idx >= D * E) return;
+  const int c0 = request_chunks[b], c1 = request_chunks[b + 1];
+  if (c0 >= c1) return;
+  const int d = idx / E;
+  float* own = state + (static_cast<int64_t>(state_slots[b]) * H + head) * D * E + idx;
+  const int64_t stride = static_cast<int64_t>(H) * D * E;
+  float* p = scratch + (static_cast<int64_t>(c0) * H + head) * D * E + idx;
+  const float* g = totals + (static_cast<int64_t>(c0) * H + head) * D + d;
+  float S = *own;
+  for (int c = c0; c < c1; c += 4) {
+    // the sums of four chunks are asked for together; each then gives way to the state in front of its chunk
+    float add[4], keep[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      add[u] = c + u < c1 ? p[u * stride] : 0.f;
+      keep[u] = c + u < c1 ? g[static_cast<int64_t>(u) * H * D] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (c + u >= c1) break;
+      p[u * stride] = S;
+      S = keep[u] * S + add[u];
+    }
+    p += 4 * stride;
+    g += 4 * static_cast<int64_t>(H) * D;
+  }
+  *own = S;
+}
+
+template <typename X>
+__global__ void __launch_bounds__(256)
+gated_chunk_outputs_kernel(const X* __restrict__ product, int64_t ld, const float* __restrict__ logits, float tau,
+                           float q_scale, const float* __restrict__ scratch, float* __restrict__ out,
+                           const int4* __restrict__ chunks, int H, int D, int E) {
+  extern __shared__ float lds[];
+  float* Ct = lds;                        // [D][68]: Ct[d][i] = c_i[d]
+  float* Qt = Ct + D * GS_PAD;            // [D][68]: q_i[d] * q_scale; behind the scores, times exp(c_i[d])
+  float* Kt = Qt + D * GS_PAD;            // [D][68]; behind the scores, the state in front of the chunk [D][64]
+  float* At = Kt + D * GS_PAD;            // [64][68]: At[j][i] = sum_d q_i[d] k_j[d] exp(c_i[d] - c_j[d]) for j <= i
+  float* Vs = At + GS_L * GS_PAD;         // [64][64]
+  const int c = blockIdx.x, head = blockIdx.y, e0 = blockIdx.z * 64;
+  const int4 chunk = chunks[c];
+  const int64_t row0 = chunk.y;
+  const int len = chunk.z;
+  decay_prefix(Ct, logits, row0, len, head, H, D, tau);
+  for (int idx = threadIdx.x; idx < GS_L * D; idx += blockDim.x) {
+    const int j = idx / D, d = idx % D;
+    const X* row = product + (row0 + j) * ld;
+    Qt[d * GS_PAD + j] = j < len ? to_float(row[head * D + d]) * q_scale : 0.f;
+    Kt[d * GS_PAD + j] = j < len ? to_float(row[(H + head) * D + d]) : 0.f;
+  }
+  for (int idx = threadIdx.x; idx < GS_L * 64; idx += blockDim.x) {
+    const int j = idx / 64, col = idx % 64;
+    Vs[idx] = (j < len && e0 + col < E) ? to_float(product[(row0 + j) * ld + 2 * H * D + head * E + e0 + col]) : 0.f;
+  }
+  __syncthreads();
+  const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+  float s4[4][4] = {};
+  if (tx <= ty) {
+#pragma unroll 2
+    for (int d = 0; d < D; ++d) {
+      const float4 q4 = *reinterpret_cast<const float4*>(Qt + d * GS_PAD + 4 * ty);
+      const float4 k4 = *reinterpret_cast<const float4*>(Kt + d * GS_PAD + 4 * tx);
+      const float4 i4 = *reinterpret_cast<const float4*>(Ct + d * GS_PAD + 4 * ty);
+      const float4 j4 = *reinterpret_cast<const float4*>(Ct + d * GS_PAD + 4 * tx);
+      const float q[4] = {q4.x, q4.y, q4.z, q4.w}, k[4] = {k4.x, k4.y, k4.z, k4.w};
+      const float ci[4] = {i4.x, i4.y, i4.z, i4.w}, cj[4] = {j4.x, j4.y, j4.z, j4.w};
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) s4[a][b] += q[a] * k[b] * expf(fminf(ci[a] - cj[b], 0.f));
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int i = 4 * ty + a, j = 4 * tx + b;
+      At[j * GS_PAD + i] = j <= i ? s4[a][b] : 0.f;
+    }
+  __syncthreads();
+  float* Ss = Kt;
+  const float* src = scratch + (static_cast<int64_t>(c) * H + head) * D * E;
+  for (int idx = threadIdx.x; idx < D * 64; idx += blockDim.x) {
+    const int d = idx / 64, col = idx % 64;
+    Ss[idx] = e0 + col < E ? src[static_cast<int64_t>(d) * E + e0 + col] : 0.f;
+  }
+  for (int idx = threadIdx.x; idx < GS_L * D; idx += blockDim.x) {
+    const int j = idx % GS_L, d = idx / GS_L;
+    Qt[d * GS_PAD + j] *= expf(Ct[d * GS_PAD + j]);
+  }
+  __syncthreads();
+  float o[4][4] = {};
+#pragma unroll 8
+  for (int d = 0; d < D; ++d) {
+    const float4 q4 = *reinterpret_cast<const float4*>(Qt + d * GS_PAD + 4 * ty);
+    const float4 t4 = *reinterpret_cast<const float4*>(Ss + d * 64 + 4 * tx);
+    const float q[4] = {q4.x, q4.y, q4.z, q4.w}, t[4] = {t4.x, t4.y, t4.z, t4.w};
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) o[a][b] += q[a] * t[b];
+  }
+  const int reach = min(len, 4 * ty + 4);
+#pragma unroll 4
+  for (int j = 0; j < reach; ++j) {
+    const float4 a4 = *reinterpret_cast<const float4*>(At + j * GS_PAD + 4 * ty);
+    const float4 v4 = *reinterpret_cast<const float4*>(Vs + j * 64 + 4 * tx);
+    const float w[4] = {a4.x, a4.y, a4.z, a4.w}, v[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) o[a][b] += w[a] * v[b];
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int i = 4 * ty + a;
+    if (i >= len) continue;
+    const int e = e0 + 4 * tx;
+    if (e < E)
+      *reinterpret_cast<float4*>(out + ((row0 + i) * H + head) * E + e) = float4{o[a][0], o[a][1], o[a][2], o[a][3]};
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
 // The gates of a real-gated linear recurrent unit. u [T, ldu] holds R channels in B parts of n; in part b
 //   r = sigmoid(ra[b] u_b + ra_b[b]),  i = sigmoid(ri[b] u_b + ri_b[b])          (ra[b], ri[b]: [n, n], [out, in])
 //   a = exp(-rate * r * softplus(lam)),  x = sqrt(1 - a^2) * i * u     -> a_out, x_out float32 [T, R]
@@ -254,6 +474,78 @@ __global__ void lru_scan_kernel(const float* __restrict__ a, const float* __rest
     }
   }
   *own = h;
+}
+
+// The same scan over portions of prompts in chunks of rows that run side by side: every chunk first alone from
+// h = 0 (its last value X and the product A of its factors), then again from the value in front of it, which a thread
+// gets by walking the request's earlier chunks, h <- A h + X. The request's first chunk hands the state in front of
+// the step to `init`, so that the last chunk may write the state behind it while others still read.
+constexpr int LS_ROWS = 64;
+
+__global__ void lru_chunk_sums_kernel(const float* __restrict__ a, const float* __restrict__ x, const float* __restrict__ state,
+                                      float* __restrict__ factors, float* __restrict__ sums, float* __restrict__ init,
+                                      const int4* __restrict__ chunks, const int32_t* __restrict__ request_chunks,
+                                      const int32_t* __restrict__ state_slots, int R) {
+  const int chunk = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= R) return;
+  const int4 entry = chunks[chunk];
+  const int64_t row0 = entry.y;
+  const int len = entry.z;
+  if (request_chunks[entry.x] == chunk) init[static_cast<int64_t>(entry.x) * R + c] = state[static_cast<int64_t>(state_slots[entry.x]) * R + c];
+  float A = 1.f, X = 0.f;
+  for (int j = 0; j < len; j += 4) {
+    float av[4], xv[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int64_t r = row0 + min(j + k, len - 1);
+      av[k] = a[r * R + c];
+      xv[k] = x[r * R + c];
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (j + k >= len) break;
+      X = av[k] * X + xv[k];
+      A *= av[k];
+    }
+  }
+  factors[static_cast<int64_t>(chunk) * R + c] = A;
+  sums[static_cast<int64_t>(chunk) * R + c] = X;
+}
+
+template <typename M, typename O>
+__global__ void lru_chunk_apply_kernel(const float* __restrict__ a, const float* __restrict__ x, float* __restrict__ state,
+                                       const float* __restrict__ factors, const float* __restrict__ sums,
+                                       const float* __restrict__ init, const M* __restrict__ mul, int64_t ldm, int kind,
+                                       O* __restrict__ out, const int4* __restrict__ chunks,
+                                       const int32_t* __restrict__ request_chunks, const int32_t* __restrict__ state_slots,
+                                       int R) {
+  const int chunk = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= R) return;
+  const int4 entry = chunks[chunk];
+  const int64_t row0 = entry.y;
+  const int len = entry.z;
+  float h = init[static_cast<int64_t>(entry.x) * R + c];
+  for (int before = request_chunks[entry.x]; before < chunk; ++before)
+    h = factors[static_cast<int64_t>(before) * R + c] * h + sums[static_cast<int64_t>(before) * R + c];
+  for (int j = 0; j < len; j += 4) {
+    float av[4], xv[4], mv[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int64_t r = row0 + min(j + k, len - 1);
+      av[k] = a[r * R + c];
+      xv[k] = x[r * R + c];
+      mv[k] = mul != nullptr ? to_float(mul[r * ldm + c]) : 1.f;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (j + k >= len) break;
+      h = av[k] * h + xv[k];
+      out[(row0 + j + k) * R + c] = from_float<O>(mul != nullptr ? h * activate(mv[k], kind) : h);
+    }
+  }
+  if (chunk + 1 == request_chunks[entry.x + 1]) state[static_cast<int64_t>(state_slots[entry.x]) * R + c] = h;
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -378,6 +670,48 @@ extern "C" int distie_gated_decay_scan(const void* product, int dtype, int64_t l
   return launch_status();
 }
 
+extern "C" int distie_gated_decay_scan_chunk_rows() { return GS_L; }
+// the largest per-head key size the chunked scan takes (its tiles must fit the LDS of a compute unit)
+extern "C" int distie_gated_decay_scan_chunked_max_dim() { return 128; }
+
+template <typename K>
+static int more_lds(K kernel, size_t lds) {
+  if (lds <= 48 * 1024) return 0;
+  return static_cast<int>(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              static_cast<int>(lds)));
+}
+
+// chunks: int32 [num_chunks][4] = {request, first row, rows (1..64), 0}, the chunks of a request one after the other;
+// request_chunks: int32 [B + 1], the first chunk of every request; scratch: float32 [num_chunks, H, D, E];
+// totals: float32 [num_chunks, H, D]
+extern "C" int distie_gated_decay_scan_chunked(const void* product, int dtype, int64_t ld, const float* logits,
+                                               float* state, float* out, float* scratch, float* totals,
+                                               const int32_t* chunks, const int32_t* request_chunks,
+                                               const int32_t* state_slots, int num_chunks, int B, int H, int D, int E,
+                                               float q_scale, float tau, hipStream_t stream) {
+  if (B <= 0 || num_chunks <= 0) return 0;
+  if (H < 1 || D < 4 || E < 4 || D % 4 || E % 4 || D > 128 || !(tau > 0.f) || ld < static_cast<int64_t>(H) * (2 * D + E))
+    return DISTIE_BAD_ARGUMENT;
+  const dim3 grid(num_chunks, H, (E + 63) / 64);
+  const int4* table = reinterpret_cast<const int4*>(chunks);
+  const size_t lds_sums = (static_cast<size_t>(D) * GS_PAD + GS_L * D + GS_L * 64) * sizeof(float);
+  const size_t lds_out = (3 * static_cast<size_t>(D) * GS_PAD + GS_L * GS_PAD + GS_L * 64) * sizeof(float);
+  int status = 0;
+  DISTIE_DISPATCH(dtype, X, {
+    if ((status = more_lds(gated_chunk_sums_kernel<X>, lds_sums)) != 0) return status;
+    if ((status = more_lds(gated_chunk_outputs_kernel<X>, lds_out)) != 0) return status;
+    gated_chunk_sums_kernel<X><<<grid, 256, lds_sums, stream>>>(static_cast<const X*>(product), ld, logits, tau, scratch,
+                                                                totals, table, H, D, E);
+    if ((status = launch_status()) != 0) return status;
+    gated_chunk_states_kernel<<<dim3(B, H, (D * E + 255) / 256), 256, 0, stream>>>(scratch, totals, state, request_chunks,
+                                                                                  state_slots, H, D, E);
+    if ((status = launch_status()) != 0) return status;
+    gated_chunk_outputs_kernel<X><<<grid, 256, lds_out, stream>>>(static_cast<const X*>(product), ld, logits, tau, q_scale,
+                                                                  scratch, out, table, H, D, E);
+  });
+  return launch_status();
+}
+
 extern "C" int distie_lru_gates(const void* u, int u_dtype, int64_t ldu, const void* ra, const float* ra_b, const void* ri,
                                 const float* ri_b, int w_dtype, const float* lam, float rate, float* a_out, float* x_out,
                                 int T, int R, int blocks, hipStream_t stream) {
@@ -403,6 +737,29 @@ extern "C" int distie_lru_scan(const float* a, const float* x, float* state, con
   DISTIE_DISPATCH(mul_dtype, M, DISTIE_DISPATCH(out_dtype, O,
       lru_scan_kernel<M, O><<<grid, threads, 0, stream>>>(a, x, state, static_cast<const M*>(mul), ldm, kind,
                                                           static_cast<O*>(out), cu_q, state_slots, R)));
+  return launch_status();
+}
+
+extern "C" int distie_lru_scan_chunk_rows() { return LS_ROWS; }
+
+// chunks / request_chunks as for the chunked scans of states; factors, sums: float32 [num_chunks, R]; init: float32 [B, R]
+extern "C" int distie_lru_scan_chunked(const float* a, const float* x, float* state, float* factors, float* sums, float* init,
+                                       const void* mul, int mul_dtype, int64_t ldm, int kind, void* out, int out_dtype,
+                                       const int32_t* chunks, const int32_t* request_chunks, const int32_t* state_slots,
+                                       int num_chunks, int B, int R, hipStream_t stream) {
+  if (B <= 0 || num_chunks <= 0) return 0;
+  if (R < 1 || kind < -1 || kind > 3 || (mul != nullptr && ldm < R)) return DISTIE_BAD_ARGUMENT;
+  if (mul == nullptr) mul_dtype = DISTIE_F32;
+  const int threads = R >= 256 ? 256 : (R >= 128 ? 128 : 64);
+  const dim3 grid(num_chunks, (R + threads - 1) / threads);
+  const int4* table = reinterpret_cast<const int4*>(chunks);
+  lru_chunk_sums_kernel<<<grid, threads, 0, stream>>>(a, x, state, factors, sums, init, table, request_chunks, state_slots, R);
+  const int status = launch_status();
+  if (status != 0) return status;
+  DISTIE_DISPATCH(mul_dtype, M, DISTIE_DISPATCH(out_dtype, O,
+      lru_chunk_apply_kernel<M, O><<<grid, threads, 0, stream>>>(a, x, state, factors, sums, init,
+                                                                 static_cast<const M*>(mul), ldm, kind, static_cast<O*>(out),
+                                                                 table, request_chunks, state_slots, R)));
   return launch_status();
 }
 

@@ -313,8 +313,10 @@ class HipOps(Ops):
         o.distie_rmsnorm_gate.argtypes = [_P, _P, _I, _F, _P, _I, _L, _P, _I, _I, _I, _I, _I, _P]
         o.distie_norm_chain.argtypes = [_P, _I, _I, _P, _P, _I, _I, _P, _F, _F, _P, _F, _P, _P, _F, _P, _I, _P, _I, _I, _P]
         o.distie_gated_decay_scan.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _P]
+        o.distie_gated_decay_scan_chunked.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P]
         o.distie_lru_gates.argtypes = [_P, _I, _L, _P, _P, _P, _P, _I, _P, _F, _P, _P, _I, _I, _I, _P]
         o.distie_lru_scan.argtypes = [_P, _P, _P, _P, _I, _L, _I, _P, _I, _P, _P, _I, _I, _P]
+        o.distie_lru_scan_chunked.argtypes = [_P, _P, _P, _P, _P, _P, _P, _I, _L, _I, _P, _I, _P, _P, _P, _I, _I, _I, _P]
         o.distie_route_topk.argtypes = [_P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _P]
         o.distie_route_scale.argtypes = [_P, _I, _L, _P, _P, _I, _I, _I, _I, _P]
         o.distie_scale_f32.argtypes = [_P, _L, _F, _P]
@@ -1042,6 +1044,7 @@ class HipOps(Ops):
     # a step in which some request brings at least so many rows runs the decayed state in chunks of rows that are
     # worked side by side (three kernels) instead of row after row (one)
     SCAN_CHUNKED_MIN_ROWS = 16
+    LRU_CHUNKED_MIN_ROWS = 128       # the same for the scan of a channel-wise recurrence (chunks of 64 rows, two kernels)
     ACTIVATIONS = {"relu2": 0, "silu": 1, "gelu_tanh": 2, "relu": 3}
 
     def hyper_step(self, streams, *, init=None, delta=None, gate=None, mix=None, write=None, read=None,
@@ -1186,6 +1189,30 @@ class HipOps(Ops):
                "sigmoid_gate")
         return out
 
+    def _scan_chunks(self, meta, rows, num_heads, dim, value_dim):
+        """Which rows of the step form a chunk of a state's scan, worked out from the step's row counts (known on the
+        host outside captured steps): (number of chunks, the table {request, first row, rows, 0} with the first chunk
+        of every request behind it, scratch for a state a chunk)."""
+        table_key = ("scan_chunk_table", rows)
+        held = meta.scratch.get(table_key)
+        if held is None:
+            cu = np.asarray(meta.host_cu_q, dtype=np.int64)
+            table, first = [], [0]
+            for b in range(meta.num_requests):
+                for at in range(int(cu[b]), int(cu[b + 1]), rows):
+                    table.append((b, at, min(rows, int(cu[b + 1]) - at), 0))
+                first.append(len(table))
+            packed = self.upload(np.concatenate([np.asarray(table, dtype=np.int32).reshape(-1),
+                                                 np.asarray(first, dtype=np.int32)]))
+            held = meta.scratch[table_key] = (len(table), packed)
+        count, packed = held
+        key = ("scan_chunks", rows, num_heads, dim, value_dim)
+        scratch = meta.scratch.get(key)
+        if scratch is None:
+            scratch = meta.scratch[key] = torch.empty((count, num_heads, dim, value_dim), dtype=torch.float32,
+                                                      device=self.device)
+        return count, packed, scratch
+
     def decay_scan(self, product, state, decay, meta, num_heads, dim, value_dim):
         product = self.dense(product)
         self._own(product, state, decay)
@@ -1201,21 +1228,8 @@ class HipOps(Ops):
                 dim % 4 == 0 and value_dim % 4 == 0 and dim <= self._ops.distie_decay_scan_chunked_max_dim():
             # portions of prompts: chunks of rows side by side instead of one row after the other. Which rows form
             # a chunk is worked out here from the step's row counts (known on the host outside captured steps).
-            key = ("scan_chunks", num_heads, dim, value_dim)
-            plan = meta.scratch.get(key)
-            if plan is None:
-                rows = self._ops.distie_decay_scan_chunk_rows()
-                cu = np.asarray(meta.host_cu_q, dtype=np.int64)
-                table, first = [], [0]
-                for b in range(meta.num_requests):
-                    for at in range(int(cu[b]), int(cu[b + 1]), rows):
-                        table.append((b, at, min(rows, int(cu[b + 1]) - at), 0))
-                    first.append(len(table))
-                packed = self.upload(np.concatenate([np.asarray(table, dtype=np.int32).reshape(-1),
-                                                     np.asarray(first, dtype=np.int32)]))
-                scratch = torch.empty((len(table), num_heads, dim, value_dim), dtype=torch.float32, device=self.device)
-                plan = meta.scratch[key] = (len(table), packed, scratch)
-            count, packed, scratch = plan
+            count, packed, scratch = self._scan_chunks(meta, self._ops.distie_decay_scan_chunk_rows(), num_heads, dim,
+                                                       value_dim)
             _check(self._ops.distie_decay_scan_chunked(
                 product.data_ptr(), _code(product), W, state.data_ptr(), decay.data_ptr(), out.data_ptr(),
                 scratch.data_ptr(), packed.data_ptr(), packed.data_ptr() + 16 * count, meta.state_slots.data_ptr(),
@@ -1328,6 +1342,19 @@ class HipOps(Ops):
         if state.dtype != torch.float32 or tuple(state.shape[1:]) != (num_heads, dim, value_dim):
             raise KernelError("gated_decay_scan: the state is float32 [slots, heads, dim, value_dim]")
         out = torch.empty((T, num_heads * value_dim), dtype=torch.float32, device=self.device)
+        if not self.captured and meta.host_cu_q is not None and meta.max_q >= self.SCAN_CHUNKED_MIN_ROWS and \
+                dim % 4 == 0 and value_dim % 4 == 0 and dim <= self._ops.distie_gated_decay_scan_chunked_max_dim():
+            # portions of prompts: chunks of rows side by side instead of one row after the other
+            count, packed, scratch = self._scan_chunks(meta, self._ops.distie_gated_decay_scan_chunk_rows(), num_heads,
+                                                       dim, value_dim)
+            totals = torch.empty((count, num_heads, dim), dtype=torch.float32, device=self.device)
+            _check(self._ops.distie_gated_decay_scan_chunked(
+                product.data_ptr(), _code(product), W, decay_logits.data_ptr(), state.data_ptr(), out.data_ptr(),
+                scratch.data_ptr(), totals.data_ptr(), packed.data_ptr(), packed.data_ptr() + 16 * count,
+                meta.state_slots.data_ptr(), count, meta.num_requests, num_heads, dim, value_dim, float(q_scale),
+                float(tau), self._stream()), "gated_decay_scan_chunked")
+            _mark_written(state)
+            return out
         _check(self._ops.distie_gated_decay_scan(
             product.data_ptr(), _code(product), W, decay_logits.data_ptr(), state.data_ptr(), out.data_ptr(),
             meta.cu_q.data_ptr(), meta.state_slots.data_ptr(), meta.num_requests, num_heads, dim, value_dim,
@@ -1373,6 +1400,17 @@ class HipOps(Ops):
             m_ptr, m_ld = self._rows_view(mul, R)
             m_code = _code(mul)
         out = torch.empty((T, R), dtype=out_dtype, device=self.device)
+        if not self.captured and meta.host_cu_q is not None and meta.max_q >= self.LRU_CHUNKED_MIN_ROWS:
+            # portions of prompts: chunks of rows side by side, each scanned twice (alone, then from what stands before it)
+            count, packed, sums = self._scan_chunks(meta, self._ops.distie_lru_scan_chunk_rows(), 1, 1, R)
+            factors = torch.empty((count, R), dtype=torch.float32, device=self.device)
+            init = torch.empty((meta.num_requests, R), dtype=torch.float32, device=self.device)
+            _check(self._ops.distie_lru_scan_chunked(
+                a.data_ptr(), x.data_ptr(), state.data_ptr(), factors.data_ptr(), sums.data_ptr(), init.data_ptr(), m_ptr,
+                m_code, m_ld, kind, out.data_ptr(), _code(out), packed.data_ptr(), packed.data_ptr() + 16 * count,
+                meta.state_slots.data_ptr(), count, meta.num_requests, R, self._stream()), "lru_scan_chunked")
+            _mark_written(state)
+            return out
         _check(self._ops.distie_lru_scan(a.data_ptr(), x.data_ptr(), state.data_ptr(), m_ptr, m_code, m_ld, kind,
                                          out.data_ptr(), _code(out), meta.cu_q.data_ptr(), meta.state_slots.data_ptr(),
                                          meta.num_requests, R, self._stream()), "lru_scan")

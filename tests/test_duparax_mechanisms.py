@@ -161,9 +161,12 @@ def test_norm_of_every_head_with_a_silu_gate(ops):
 
 @pytest.mark.parametrize("lengths,cuts", [(LENGTHS, CUTS), (LONG_LENGTHS, LONG_CUTS)])
 @pytest.mark.parametrize("width,blocks,taps", [(64, 4, 4), (40, 4, 3), (48, 1, 1), (32, 32, 2), (200, 2, 2)])
-def test_recurrent_unit(ops, width, blocks, taps, lengths, cuts):
+def test_recurrent_unit(ops, width, blocks, taps, lengths, cuts, monkeypatch):
     """Convolution with a bias on a view of columns, block-diagonal gates, the recurrence and the product with the
-    other branch, with the inputs and the state handed from step to step."""
+    other branch, with the inputs and the state handed from step to step. Long portions go through the scan in
+    chunks of rows (on the GPU)."""
+    if hasattr(ops, "LRU_CHUNKED_MIN_ROWS"):
+        monkeypatch.setattr(ops, "LRU_CHUNKED_MIN_ROWS", 16)
     R, n = width, width // blocks
     for dtype in act_types(ops):
         conv, conv_b = rnd(R, taps, seed=1, scale=0.5).to(dtype), rnd(R, seed=2, scale=0.3)
