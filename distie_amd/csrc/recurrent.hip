@@ -33,59 +33,170 @@ __device__ __forceinline__ float activate(float z, int kind) {   // the kinds of
 //   x  += y                                          (residual, float32, in place; null: y goes to y_out)
 //   out = rms(x) * pre_w                             (the norm in front of the next sub-layer)
 // rms(v) = v / sqrt(mean(v^2) + eps). A term may be partial sums (slices that lie `stride` apart, added in order).
-// The row waits in LDS between the passes; a thread meets the same columns in every pass.
-template <typename A, typename B, typename O>
+// The row waits in LDS between the passes; a thread meets the same columns in every pass. `held`: the terms and the
+// residual are read once, up front and together, and wait in LDS too (rows of up to NORM_HELD_MAX columns); else
+// they are read again where they are needed.
+constexpr int NORM_HELD_MAX = 8192;
+
+// V values at p as floats: V = 4 takes one 16-byte (float32) or 8-byte (bfloat16) load
+template <int V, typename T>
+__device__ __forceinline__ void load_values(const T* __restrict__ p, float out[V]) {
+  if constexpr (V == 4 && sizeof(T) == 4) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    out[0] = v.x, out[1] = v.y, out[2] = v.z, out[3] = v.w;
+  } else if constexpr (V == 4) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    out[0] = __uint_as_float(v.x << 16), out[1] = __uint_as_float(v.x & 0xffff0000u);
+    out[2] = __uint_as_float(v.y << 16), out[3] = __uint_as_float(v.y & 0xffff0000u);
+  } else {
+#pragma unroll
+    for (int k = 0; k < V; ++k) out[k] = to_float(p[k]);
+  }
+}
+
+template <int V, typename T>
+__device__ __forceinline__ void store_values(T* __restrict__ p, const float v[V]) {
+  if constexpr (V == 4 && sizeof(T) == 4) {
+    *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
+  } else if constexpr (V == 4) {
+    const auto word = [](float lo, float hi) {
+      return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(lo))) |
+             (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(hi))) << 16);
+    };
+    *reinterpret_cast<uint2*>(p) = uint2{word(v[0], v[1]), word(v[2], v[3])};
+  } else {
+#pragma unroll
+    for (int k = 0; k < V; ++k) p[k] = from_float<T>(v[k]);
+  }
+}
+
+// the sum of `slices` vectors that lie `stride` elements apart, added in order; eight slices' loads under way together
+template <int V, typename T>
+__device__ __forceinline__ void sum_values(const T* __restrict__ p, int slices, int64_t stride, float out[V]) {
+  load_values<V>(p, out);
+  for (int s = 1; s < slices; s += 8) {
+    float a[8][V];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) load_values<V>(p + min(s + u, slices - 1) * stride, a[u]);
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (s + u < slices) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) out[k] += a[u][k];
+      }
+  }
+}
+
+template <int V, typename A, typename B, typename O>
 __global__ void norm_chain_kernel(const A* __restrict__ t0, int slices0, int64_t stride0, const float* __restrict__ w0,
                                   const B* __restrict__ t1, int slices1, int64_t stride1, const float* __restrict__ w1,
                                   float term_eps, float scale, const float* __restrict__ post_w, float post_eps,
                                   float* __restrict__ residual, const float* __restrict__ pre_w, float pre_eps,
-                                  O* __restrict__ out, float* __restrict__ y_out, int C) {
+                                  O* __restrict__ out, float* __restrict__ y_out, int C, int held) {
   extern __shared__ float row[];
   __shared__ float scratch[16];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * C;
+  float* held_a = row + C;
+  float* held_b = row + 2 * C;
+  float* held_x = row + 3 * C;
+  const int step = V * blockDim.x;
+  if (held) {
+    for (int c = V * threadIdx.x; c < C; c += step) {
+      float a[V], b[V] = {}, x[V] = {};
+      sum_values<V>(t0 + base + c, slices0, stride0, a);
+      if (t1 != nullptr) sum_values<V>(t1 + base + c, slices1, stride1, b);
+      if (residual != nullptr) load_values<V>(residual + base + c, x);
+      store_values<V>(held_a + c, a);
+      store_values<V>(held_b + c, b);
+      store_values<V>(held_x + c, x);
+    }
+  }
   float r0 = 1.f, r1 = 1.f;
   if (w0 != nullptr) {
     float q0 = 0.f, q1 = 0.f;
-    for (int c = threadIdx.x; c < C; c += blockDim.x) {
-      const float a = sum_strided(t0 + base + c, slices0, stride0);
-      q0 += a * a;
-      if (t1 != nullptr) {
-        const float b = sum_strided(t1 + base + c, slices1, stride1);
-        q1 += b * b;
+    for (int c = V * threadIdx.x; c < C; c += step) {
+      float a[V], b[V] = {};
+      if (held) {
+        load_values<V>(held_a + c, a);
+        load_values<V>(held_b + c, b);
+      } else {
+        sum_values<V>(t0 + base + c, slices0, stride0, a);
+        if (t1 != nullptr) sum_values<V>(t1 + base + c, slices1, stride1, b);
       }
+#pragma unroll
+      for (int k = 0; k < V; ++k) q0 += a[k] * a[k], q1 += b[k] * b[k];
     }
     r0 = 1.f / sqrtf(block_sum(q0, scratch) / C + term_eps);
     if (t1 != nullptr) r1 = 1.f / sqrtf(block_sum(q1, scratch) / C + term_eps);
   }
   float q = 0.f;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float y = sum_strided(t0 + base + c, slices0, stride0);
-    if (w0 != nullptr) {
-      y = y * r0 * w0[c];
-      if (t1 != nullptr) y += sum_strided(t1 + base + c, slices1, stride1) * r1 * w1[c];
-      y *= scale;
+  for (int c = V * threadIdx.x; c < C; c += step) {
+    float y[V];
+    if (held) {
+      load_values<V>(held_a + c, y);
+    } else {
+      sum_values<V>(t0 + base + c, slices0, stride0, y);
     }
-    row[c] = y;
-    q += y * y;
+    if (w0 != nullptr) {
+      float w[V];
+      load_values<V>(w0 + c, w);
+#pragma unroll
+      for (int k = 0; k < V; ++k) y[k] = y[k] * r0 * w[k];
+      if (t1 != nullptr) {
+        float b[V];
+        if (held) {
+          load_values<V>(held_b + c, b);
+        } else {
+          sum_values<V>(t1 + base + c, slices1, stride1, b);
+        }
+        load_values<V>(w1 + c, w);
+#pragma unroll
+        for (int k = 0; k < V; ++k) y[k] += b[k] * r1 * w[k];
+      }
+#pragma unroll
+      for (int k = 0; k < V; ++k) y[k] *= scale;
+    }
+    store_values<V>(row + c, y);
+#pragma unroll
+    for (int k = 0; k < V; ++k) q += y[k] * y[k];
   }
   float rp = 1.f;
   if (post_w != nullptr) rp = 1.f / sqrtf(block_sum(q, scratch) / C + post_eps);
   float q2 = 0.f;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float y = row[c];
-    if (post_w != nullptr) y = y * rp * post_w[c];
+  for (int c = V * threadIdx.x; c < C; c += step) {
+    float y[V];
+    load_values<V>(row + c, y);
+    if (post_w != nullptr) {
+      float w[V];
+      load_values<V>(post_w + c, w);
+#pragma unroll
+      for (int k = 0; k < V; ++k) y[k] = y[k] * rp * w[k];
+    }
     if (residual != nullptr) {
-      const float x = residual[base + c] + y;
-      residual[base + c] = x;
-      row[c] = x;
-      q2 += x * x;
+      float x[V];
+      if (held) {
+        load_values<V>(held_x + c, x);
+      } else {
+        load_values<V>(residual + base + c, x);
+      }
+#pragma unroll
+      for (int k = 0; k < V; ++k) x[k] += y[k], q2 += x[k] * x[k];
+      store_values<V>(residual + base + c, x);
+      store_values<V>(row + c, x);
     } else {
-      y_out[base + c] = y;
+      store_values<V>(y_out + base + c, y);
     }
   }
   if (residual == nullptr || pre_w == nullptr) return;
   const float rn = 1.f / sqrtf(block_sum(q2, scratch) / C + pre_eps);
-  for (int c = threadIdx.x; c < C; c += blockDim.x) out[base + c] = from_float<O>(row[c] * rn * pre_w[c]);
+  for (int c = V * threadIdx.x; c < C; c += step) {
+    float x[V], w[V];
+    load_values<V>(row + c, x);
+    load_values<V>(pre_w + c, w);
+#pragma unroll
+    for (int k = 0; k < V; ++k) x[k] = x[k] * rn * w[k];
+    store_values<V>(out + base + c, x);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -327,7 +438,11 @@ gated_chunk_outputs_kernel(const X* __restrict__ product, int64_t ld, const floa
 #pragma unroll
       for (int a = 0; a < 4; ++a)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) s4[a][b] += q[a] * k[b] * expf(fminf(ci[a] - cj[b], 0.f));
+        for (int b = 0; b < 4; ++b) {
+          // (bfloat16 steps take the hardware's exponent: their q and k carry eight bits)
+          const float x = fminf(ci[a] - cj[b], 0.f);
+          s4[a][b] += q[a] * k[b] * (sizeof(X) == 2 ? __expf(x) : expf(x));
+        }
     }
   }
 #pragma unroll
@@ -441,6 +556,54 @@ lru_gates_kernel(const X* __restrict__ u, int64_t ldu, const W* __restrict__ ra,
     const float log_a = decay * r;
     a_out[static_cast<int64_t>(t) * R + c] = expf(log_a);
     x_out[static_cast<int64_t>(t) * R + c] = sqrtf(-expm1f(2.f * log_a)) * i * to_float(u[static_cast<int64_t>(t) * ldu + c]);
+  }
+}
+
+// The same for steps of up to LG_FEW rows: a wave owns one output channel, its lanes share the inputs of the part; both
+// weight rows and every row's inputs are asked for before the first is used, so a step waits for one trip to memory.
+constexpr int LG_FEW = 8;
+
+template <typename X, typename W>
+__global__ void __launch_bounds__(256)
+lru_gates_few_kernel(const X* __restrict__ u, int64_t ldu, const W* __restrict__ ra, const float* __restrict__ ra_b,
+                     const W* __restrict__ ri, const float* __restrict__ ri_b, const float* __restrict__ lam, float rate,
+                     float* __restrict__ a_out, float* __restrict__ x_out, int T, int R, int n) {
+  const int lane = threadIdx.x % 64;
+  const int c = blockIdx.x * 4 + threadIdx.x / 64;
+  if (c >= R) return;
+  const int part = c / n;
+  const W* wa = ra + static_cast<int64_t>(c) * n;          // [part][c - part * n][:] is row c of the stacked blocks
+  const W* wi = ri + static_cast<int64_t>(c) * n;
+  float acc_a[LG_FEW] = {}, acc_i[LG_FEW] = {};
+  const float bias_a = ra_b[c], bias_i = ri_b[c], lam_c = lam[c];
+  const float self = lane < T ? to_float(u[static_cast<int64_t>(lane) * ldu + c]) : 0.f;     // lane t: row t's own input
+  for (int k0 = lane; k0 < n; k0 += 64 * 2) {
+    float a[2], i[2], x[2][LG_FEW];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int k = k0 + 64 * s;
+      a[s] = k < n ? to_float(wa[k]) : 0.f;
+      i[s] = k < n ? to_float(wi[k]) : 0.f;
+#pragma unroll
+      for (int t = 0; t < LG_FEW; ++t) x[s][t] = (k < n && t < T) ? to_float(u[static_cast<int64_t>(t) * ldu + part * n + k]) : 0.f;
+    }
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int t = 0; t < LG_FEW; ++t) acc_a[t] += a[s] * x[s][t], acc_i[t] += i[s] * x[s][t];
+  }
+  float sum_a = 0.f, sum_i = 0.f;                      // lane t: row t's sums
+#pragma unroll
+  for (int t = 0; t < LG_FEW; ++t) {
+    if (t >= T) break;
+    const float sa = wave_sum(acc_a[t]), si = wave_sum(acc_i[t]);
+    if (lane == t) sum_a = sa, sum_i = si;
+  }
+  if (lane < T) {
+    const float r = sigmoid_exact(sum_a + bias_a), i = sigmoid_exact(sum_i + bias_i);
+    const float log_a = -rate * softplus(lam_c) * r;
+    a_out[static_cast<int64_t>(lane) * R + c] = expf(log_a);
+    x_out[static_cast<int64_t>(lane) * R + c] = sqrtf(-expm1f(2.f * log_a)) * i * self;
   }
 }
 
@@ -568,7 +731,14 @@ route_topk_kernel(const X* __restrict__ x, const W* __restrict__ weight, const f
   for (int e = wave; e < E; e += 4) {
     const W* w = weight + static_cast<int64_t>(e) * C;
     float acc = 0.f;
-    for (int c = lane; c < C; c += 64) acc += to_float(w[c]) * xs[c];
+    for (int c0 = lane; c0 < C; c0 += 64 * 8) {
+      float wv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) wv[u] = c0 + 64 * u < C ? to_float(w[c0 + 64 * u]) : 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (c0 + 64 * u < C) acc += wv[u] * xs[c0 + 64 * u];
+    }
     acc = wave_sum(acc);
     if (lane == 0) z[e] = acc + (bias != nullptr ? bias[e] : 0.f);
   }
@@ -603,6 +773,89 @@ route_topk_kernel(const X* __restrict__ x, const W* __restrict__ weight, const f
   }
 }
 
+// The same for bfloat16 rows and weights whose width is a multiple of 8: a thread takes 16-byte pieces of the token's
+// row and of every expert's weight row, all asked for together (a step of few tokens waits for one trip to memory);
+// experts in groups of 16.
+constexpr int ROUTE_GROUP = 16;
+
+__device__ __forceinline__ void unpack8(const uint4& raw, float v[8]) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    v[2 * e] = __uint_as_float(w[e] << 16);
+    v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+route_topk_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ weight, const float* __restrict__ bias,
+                       int32_t* __restrict__ experts, float* __restrict__ gates, int C, int E, int top) {
+  __shared__ float z[ROUTE_MAX_EXPERTS];
+  __shared__ float part[4][ROUTE_GROUP];
+  __shared__ float chosen[ROUTE_MAX_TOP];
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int pieces = C / 8;
+  for (int e0 = 0; e0 < E; e0 += ROUTE_GROUP) {
+    float acc[ROUTE_GROUP] = {};
+    for (int p = threadIdx.x; p < pieces; p += 256) {
+      uint4 raw[ROUTE_GROUP];
+      const uint4 mine = *reinterpret_cast<const uint4*>(x + t * C + 8 * p);
+#pragma unroll
+      for (int g = 0; g < ROUTE_GROUP; ++g)
+        raw[g] = *reinterpret_cast<const uint4*>(weight + static_cast<int64_t>(min(e0 + g, E - 1)) * C + 8 * p);
+      float xv[8];
+      unpack8(mine, xv);
+#pragma unroll
+      for (int g = 0; g < ROUTE_GROUP; ++g) {
+        float wv[8];
+        unpack8(raw[g], wv);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc[g] += wv[k] * xv[k];
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < ROUTE_GROUP; ++g) {
+      const float total = wave_sum(acc[g]);
+      if (lane == 0) part[wave][g] = total;
+    }
+    __syncthreads();
+    if (threadIdx.x < ROUTE_GROUP && e0 + threadIdx.x < E) {
+      const int e = e0 + threadIdx.x;
+      z[e] = part[0][threadIdx.x] + part[1][threadIdx.x] + part[2][threadIdx.x] + part[3][threadIdx.x] +
+             (bias != nullptr ? bias[e] : 0.f);
+    }
+    __syncthreads();
+  }
+  if (wave != 0) return;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = z[e];
+      if (v > best || (v == best && e < at)) best = v, at = e;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float other = __shfl_xor(best, o, 64);
+      const int other_at = __shfl_xor(at, o, 64);
+      if (other > best || (other == best && other_at < at)) best = other, at = other_at;
+    }
+    if (at == 0x7fffffff) at = k;
+    if (lane == 0) {
+      experts[t * top + k] = at;
+      chosen[k] = best;
+    }
+    if (at % 64 == lane) z[at] = -INFINITY;
+  }
+  if (lane == 0) {
+    const float peak = chosen[0];
+    float total = 0.f;
+    for (int k = 0; k < top; ++k) total += expf(chosen[k] - peak);
+    for (int k = 0; k < top; ++k) gates[t * top + k] = expf(chosen[k] - peak) / total;
+  }
+}
+
 // hidden [T, ld]: the columns [e * F, (e + 1) * F) of expert e times the row's weight for e, zero if e was not chosen
 template <typename X>
 __global__ void route_scale_kernel(X* __restrict__ hidden, int64_t ld, const int32_t* __restrict__ experts,
@@ -615,6 +868,31 @@ __global__ void route_scale_kernel(X* __restrict__ hidden, int64_t ld, const int
       if (experts[t * top + k] == e) g = gates[t * top + k];
     X* p = hidden + t * ld + c;
     *p = from_float<X>(to_float(*p) * g);
+  }
+}
+
+// the same on 16-byte pieces of bfloat16 rows (F, ld multiples of 8)
+__global__ void route_scale_bf16x8_kernel(bf16_t* __restrict__ hidden, int64_t ld, const int32_t* __restrict__ experts,
+                                          const float* __restrict__ gates, int top, int F, int width, int64_t T) {
+  const int width8 = width / 8;
+  const int64_t total = T * width8;
+  for (int64_t it = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; it < total;
+       it += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t t = it / width8;
+    const int c = 8 * static_cast<int>(it % width8);
+    const int e = c / F;
+    float g = 0.f;
+    for (int k = 0; k < top; ++k)
+      if (experts[t * top + k] == e) g = gates[t * top + k];
+    uint4* p = reinterpret_cast<uint4*>(hidden + t * ld + c);
+    float v[8];
+    unpack8(*p, v);
+    uint32_t w[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      w[k] = static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(v[2 * k] * g))) |
+             (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(v[2 * k + 1] * g))) << 16);
+    *p = uint4{w[0], w[1], w[2], w[3]};
   }
 }
 
@@ -636,12 +914,30 @@ extern "C" int distie_norm_chain(const void* t0, int t0_dtype, int slices0, cons
     return DISTIE_BAD_ARGUMENT;
   if (t1 == nullptr) t1_dtype = t0_dtype, slices1 = 1;
   if (out == nullptr) out_dtype = DISTIE_F32;
-  const int threads = C >= 2048 ? 512 : (C >= 512 ? 256 : (C >= 128 ? 128 : 64));
   const int64_t stride = static_cast<int64_t>(T) * C;
-  DISTIE_DISPATCH(t0_dtype, A, DISTIE_DISPATCH(t1_dtype, B, DISTIE_DISPATCH(out_dtype, O,
-      norm_chain_kernel<A, B, O><<<T, threads, static_cast<size_t>(C) * sizeof(float), stream>>>(
-          static_cast<const A*>(t0), slices0, stride, w0, static_cast<const B*>(t1), slices1, stride, w1, term_eps, scale,
-          post_w, post_eps, residual, pre_w, pre_eps, static_cast<O*>(out), y_out, C))));
+  const int held = C <= NORM_HELD_MAX ? 1 : 0;
+  const size_t lds = static_cast<size_t>(C) * sizeof(float) * (held ? 4 : 1);
+  const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool wide = C % 4 == 0 && aligned(t0) && aligned(t1) && aligned(w0) && aligned(w1) && aligned(post_w) &&
+                    aligned(residual) && aligned(pre_w) && aligned(out) && aligned(y_out);
+  const int per = wide ? C / 4 : C;
+  const int threads = per >= 1024 ? 1024 : (per >= 512 ? 512 : (per >= 256 ? 256 : (per >= 128 ? 128 : 64)));
+#define DISTIE_NORM_CHAIN(V)                                                                                          \
+  DISTIE_DISPATCH(t0_dtype, A, DISTIE_DISPATCH(t1_dtype, B, DISTIE_DISPATCH(out_dtype, O, {                           \
+    if (lds > 48 * 1024 &&                                                                                            \
+        hipFuncSetAttribute(reinterpret_cast<const void*>(norm_chain_kernel<V, A, B, O>),                             \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)         \
+      return DISTIE_BAD_ARGUMENT;                                                                                     \
+    norm_chain_kernel<V, A, B, O><<<T, threads, lds, stream>>>(                                                       \
+        static_cast<const A*>(t0), slices0, stride, w0, static_cast<const B*>(t1), slices1, stride, w1, term_eps,     \
+        scale, post_w, post_eps, residual, pre_w, pre_eps, static_cast<O*>(out), y_out, C, held);                     \
+  })))
+  if (wide) {
+    DISTIE_NORM_CHAIN(4);
+  } else {
+    DISTIE_NORM_CHAIN(1);
+  }
+#undef DISTIE_NORM_CHAIN
   return launch_status();
 }
 
@@ -718,6 +1014,13 @@ extern "C" int distie_lru_gates(const void* u, int u_dtype, int64_t ldu, const v
   if (T <= 0) return 0;
   if (R < 1 || blocks < 1 || R % blocks || ldu < R) return DISTIE_BAD_ARGUMENT;
   const int n = R / blocks;
+  if (T <= LG_FEW) {
+    DISTIE_DISPATCH(u_dtype, X, DISTIE_DISPATCH(w_dtype, W,
+        lru_gates_few_kernel<X, W><<<(R + 3) / 4, 256, 0, stream>>>(
+            static_cast<const X*>(u), ldu, static_cast<const W*>(ra), ra_b, static_cast<const W*>(ri), ri_b, lam, rate,
+            a_out, x_out, T, R, n)));
+    return launch_status();
+  }
   const dim3 grid((T + LG_TOKENS - 1) / LG_TOKENS, blocks, (n + LG_OUT - 1) / LG_OUT);
   DISTIE_DISPATCH(u_dtype, X, DISTIE_DISPATCH(w_dtype, W,
       lru_gates_kernel<X, W><<<grid, 256, 0, stream>>>(
@@ -769,6 +1072,12 @@ extern "C" int distie_route_topk(const void* x, int x_dtype, const void* weight,
   if (C < 1 || E < 1 || E > ROUTE_MAX_EXPERTS || top < 1 || top > E || top > ROUTE_MAX_TOP ||
       static_cast<size_t>(C) * sizeof(float) > 96 * 1024)
     return DISTIE_BAD_ARGUMENT;
+  if (x_dtype == DISTIE_BF16 && w_dtype == DISTIE_BF16 && C % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(weight) % 16 == 0) {
+    route_topk_bf16_kernel<<<T, 256, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(weight), bias,
+                                                  experts, gates, C, E, top);
+    return launch_status();
+  }
   const size_t lds = static_cast<size_t>(C) * sizeof(float);
   DISTIE_DISPATCH(x_dtype, X, DISTIE_DISPATCH(w_dtype, W, {
     if (lds > 48 * 1024 &&
@@ -786,6 +1095,12 @@ extern "C" int distie_route_scale(void* hidden, int dtype, int64_t ld, const int
   if (T <= 0) return 0;
   if (top < 1 || E < 1 || F < 1 || ld < static_cast<int64_t>(E) * F) return DISTIE_BAD_ARGUMENT;
   const int width = E * F;
+  if (dtype == DISTIE_BF16 && F % 8 == 0 && ld % 8 == 0 && reinterpret_cast<uintptr_t>(hidden) % 16 == 0) {
+    const int64_t pieces = static_cast<int64_t>(T) * (width / 8);
+    const int blocks8 = static_cast<int>(pieces / 256 + 1 < 16384 ? pieces / 256 + 1 : 16384);
+    route_scale_bf16x8_kernel<<<blocks8, 256, 0, stream>>>(static_cast<bf16_t*>(hidden), ld, experts, gates, top, F, width, T);
+    return launch_status();
+  }
   const int per_row = (width + 255) / 256;
   const dim3 grid(T, per_row < 64 ? per_row : 64);
   DISTIE_DISPATCH(dtype, X, route_scale_kernel<X><<<grid, 256, 0, stream>>>(static_cast<X*>(hidden), ld, experts, gates,

@@ -86,7 +86,7 @@ def gather(seqs, rows):
     return torch.cat([seqs[i][at:at + n] for i, at, n in rows])
 
 
-@pytest.mark.parametrize("width", [40, 48, 256])
+@pytest.mark.parametrize("width", [30, 40, 48, 256, 2048])
 def test_norms_behind_sub_layers_and_normed_sums(ops, width):
     T, C = 7, width
     dev = lambda t: t.to(ops.device)
@@ -201,12 +201,13 @@ def test_router(ops, experts, top, width):
         best = torch.topk(z, top, dim=-1)
         assert chosen.dtype == torch.int32 and chosen.cpu().tolist() == best.indices.tolist()
         close(gates, torch.softmax(best.values, -1), torch.float32, "weights of the chosen")
-        hidden = rnd(T, experts * 8 + 5, seed=4).to(dtype)
-        got = ops.route_scale(hidden.clone().to(ops.device), chosen, gates, experts, 8)
         factor = torch.zeros(T, experts, dtype=F).scatter_(1, best.indices, torch.softmax(best.values, -1))
-        want = hidden.to(F).clone()
-        want[:, :experts * 8] = (want[:, :experts * 8].view(T, experts, 8) * factor[:, :, None]).view(T, -1)
-        close(got, want, dtype, "hidden values of the experts")
+        for more in (5, 16):                                      # columns behind the experts' that every row keeps
+            hidden = rnd(T, experts * 8 + more, seed=4).to(dtype)
+            got = ops.route_scale(hidden.clone().to(ops.device), chosen, gates, experts, 8)
+            want = hidden.to(F).clone()
+            want[:, :experts * 8] = (want[:, :experts * 8].view(T, experts, 8) * factor[:, :, None]).view(T, -1)
+            close(got, want, dtype, "hidden values of the experts")
     # equal logits: the lower index wins
     same = torch.zeros(2, 16)
     chosen, gates = ops.route_topk(same.to(ops.device), torch.ones(5, 16).to(ops.device), None, 2)
