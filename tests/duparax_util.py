@@ -155,9 +155,10 @@ def close_calls(cfg, weights, ids):
     """For every position, two measures of how much rounding can change what the token computes (both 1.0 where the
     model has nothing of the kind): the smallest gap between the last chosen and the first unchosen router logit over
     the routed layers, relative to the largest logit of its row; and the smallest size of a gated linear attention
-    head's output in front of its norm, relative to that head's median size over the sequence (an output near zero,
-    as the first token's is when its query and key are nearly orthogonal, comes out of the norm with a sign that
-    rounding decides). A token that is large in both is computed the same way in bfloat16."""
+    head's output in front of its norm, relative to the root of the sum of its terms' squares (what terms of random
+    signs would leave; an output that is what is left of a cancellation, as the first token's is when its query and key are
+    nearly orthogonal, comes out of the norm with a size and sign that rounding decides). A token that is large in
+    both is computed the same way in bfloat16."""
     w = {n: t.double() for n, t in weights.items()}
     eps = float(cfg["norm"]["eps"])
     T = len(ids)
@@ -173,8 +174,9 @@ def close_calls(cfg, weights, ids):
             k, v = (h @ w[r + "k"].T).view(T, H, D), (h @ w[r + "v"].T).view(T, H, E)
             z = (h @ w[r + "a1"].T) @ w[r + "a2"].T + w[r + "a2.b"]
             o = plain.gated_linear_recurrence(q, k, v, torch.sigmoid(z).pow(1.0 / float(m["tau"])).view(T, H, D))
-            size = o.pow(2).mean(-1).sqrt()
-            sizes = torch.minimum(sizes, (size / size.median(0).values).min(-1).values)
+            alpha = torch.sigmoid(z).pow(1.0 / float(m["tau"])).view(T, H, D)
+            spread = plain.gated_linear_recurrence(q ** 2, k ** 2, v ** 2, alpha ** 2)     # the terms' squares, summed
+            sizes = torch.minimum(sizes, (o.pow(2).mean(-1) / spread.mean(-1)).sqrt().min(-1).values)
             right = (plain.rms_norm(o, w[r + "norm"], eps).reshape(T, H * E) * plain.silu(h @ w[r + "g"].T)) @ w[r + "o"].T
             left = plain.left_mixer(h, w, p + "mix.left.", layer["mixer"]["left"])
             y = 0.5 * (plain.rms_norm(left, w[p + "mix.left.out"], eps) + plain.rms_norm(right, w[p + "mix.right.out"], eps))
@@ -198,7 +200,7 @@ def random_ids(cfg, n, seed):
     return torch.randint(0, cfg["vocab"], (n,), generator=torch.Generator().manual_seed(seed)).tolist()
 
 
-def clear_ids(cfg, weights, n, seed, margin=0.06, size=0.15):
+def clear_ids(cfg, weights, n, seed, margin=0.12, size=0.15):
     """`n` random token ids none of which hangs on a close call (`close_calls`): the first token that does is drawn
     again (what stands before it stays as it is, being causal), until none is left."""
     g = torch.Generator().manual_seed(seed)
