@@ -1264,9 +1264,7 @@ class HipOps(Ops):
     # ---- norms behind sub-layers, mixers side by side, gated states, routers (csrc/recurrent.hip)
     def _term(self, value):
         """(tensor, slices) of a sub-layer's result as the norm kernels read it."""
-        if isinstance(value, NormedSum):
-            value = self.dense(value)
-        if isinstance(value, (PendingNorm, PendingProduct)):
+        if isinstance(value, (NormedSum, PendingNorm, PendingProduct)):
             value = self.dense(value)
         if isinstance(value, PartialSums):
             self._own(value.data)

@@ -44,9 +44,6 @@ class ParallelMixers(Mixer):
             yield from mixer.parts()
         yield self
 
-    def capture_context(self, longest: int, limit: int):
-        return None
-
     def param_specs(self):
         return {f"{name}.out": ParamSpec((self.hidden_size,), "ones") for name in self.mixers}
 
