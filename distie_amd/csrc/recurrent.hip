@@ -205,10 +205,16 @@ __global__ void norm_chain_kernel(const A* __restrict__ t0, int slices0, int64_t
 // product [T, ld] holds q (H x D), k (H x D), v (H x E); z float32 [T, H * D]; state float32 [slots, H, D, E].
 // A block owns 64 columns e of one head of one request and walks the request's rows in order; thread (e, part)
 // keeps rows d = part, part + PARTS, ... of its column in registers, the PARTS partial sums of a column meet in LDS.
-// The next row's values are asked for before this row's are used.
-template <typename X, int PARTS, int ROWS>
+// The next row's values are asked for before this row's are used. LOW: z is not given; it is made here from `low`
+// ([T, ld_low], `rank` columns: the decay's projection through few dimensions) as z = up[h * D + d] . low + up_bias
+// (up float32 [H * D, rank], rank <= GS_RANK_MAX), which saves a step of few rows two small products.
+constexpr int GS_RANK_MAX = 32;
+
+template <typename X, int PARTS, int ROWS, bool LOW>
 __global__ void __launch_bounds__(64 * PARTS)
-gated_decay_scan_kernel(const X* __restrict__ product, int64_t ld, const float* __restrict__ logits, float* __restrict__ state,
+gated_decay_scan_kernel(const X* __restrict__ product, int64_t ld, const float* __restrict__ logits,
+                        const X* __restrict__ low, int64_t ld_low, const float* __restrict__ up,
+                        const float* __restrict__ up_bias, int rank, float* __restrict__ state,
                         float* __restrict__ out, const int32_t* __restrict__ cu_q, const int32_t* __restrict__ state_slots,
                         int H, int D, int E, float q_scale, float tau) {
   __shared__ float q_s[PARTS * ROWS], k_s[PARTS * ROWS], a_s[PARTS * ROWS];
@@ -227,12 +233,26 @@ gated_decay_scan_kernel(const X* __restrict__ product, int64_t ld, const float* 
   }
   const int d_own = threadIdx.x;                      // the channel whose q, k and decay this thread fetches
   float nq = 0.f, nk = 0.f, nz = 0.f, nv = 0.f;
+  float up_row[LOW ? GS_RANK_MAX : 1], nl[LOW ? GS_RANK_MAX : 1];
+  float bias = 0.f;
+  if constexpr (LOW) {
+    if (d_own < D) {
+      bias = up_bias[head * D + d_own];
+#pragma unroll
+      for (int r = 0; r < GS_RANK_MAX; ++r) up_row[r] = r < rank ? up[static_cast<int64_t>(head * D + d_own) * rank + r] : 0.f;
+    }
+  }
   auto fetch = [&](int t) {
     const X* row = product + static_cast<int64_t>(t) * ld;
     if (d_own < D) {
       nq = to_float(row[head * D + d_own]);
       nk = to_float(row[(H + head) * D + d_own]);
-      nz = logits[(static_cast<int64_t>(t) * H + head) * D + d_own];
+      if constexpr (LOW) {
+#pragma unroll
+        for (int r = 0; r < GS_RANK_MAX; ++r) nl[r] = r < rank ? to_float(low[static_cast<int64_t>(t) * ld_low + r]) : 0.f;
+      } else {
+        nz = logits[(static_cast<int64_t>(t) * H + head) * D + d_own];
+      }
     }
     nv = e < E ? to_float(row[2 * H * D + head * E + e]) : 0.f;
   };
@@ -240,6 +260,12 @@ gated_decay_scan_kernel(const X* __restrict__ product, int64_t ld, const float* 
   for (int t = first; t < last; ++t) {
     __syncthreads();
     if (d_own < D) {
+      if constexpr (LOW) {
+        nz = 0.f;
+#pragma unroll
+        for (int r = 0; r < GS_RANK_MAX; ++r) nz += up_row[r] * nl[r];
+        nz += bias;
+      }
       q_s[d_own] = nq * q_scale;
       k_s[d_own] = nk;
       a_s[d_own] = expf(log_sigmoid(nz) / tau);
@@ -943,16 +969,31 @@ extern "C" int distie_norm_chain(const void* t0, int t0_dtype, int slices0, cons
 
 extern "C" int distie_gated_decay_scan_max_dim() { return 256; }
 
-extern "C" int distie_gated_decay_scan(const void* product, int dtype, int64_t ld, const float* logits, float* state,
+extern "C" int distie_gated_decay_scan_max_rank() { return GS_RANK_MAX; }
+
+// logits null: z is made from low ([T, ld_low] of the product's dtype), up (float32 [H * D, rank]) and up_bias
+extern "C" int distie_gated_decay_scan(const void* product, int dtype, int64_t ld, const float* logits, const void* low,
+                                       int64_t ld_low, const float* up, const float* up_bias, int rank, float* state,
                                        float* out, const int32_t* cu_q, const int32_t* state_slots, int B, int H, int D,
                                        int E, float q_scale, float tau, hipStream_t stream) {
   if (B <= 0) return 0;
   if (H < 1 || D < 1 || E < 1 || D > 256 || !(tau > 0.f) || ld < static_cast<int64_t>(H) * (2 * D + E))
     return DISTIE_BAD_ARGUMENT;
+  if (logits == nullptr && (low == nullptr || up == nullptr || up_bias == nullptr || rank < 1 || rank > GS_RANK_MAX ||
+                            ld_low < rank))
+    return DISTIE_BAD_ARGUMENT;
   const dim3 grid(B, H, (E + 63) / 64);
 #define DISTIE_GSCAN(PARTS, ROWS)                                                                                     \
-  DISTIE_DISPATCH(dtype, X, gated_decay_scan_kernel<X, PARTS, ROWS><<<grid, 64 * PARTS, 0, stream>>>(                \
-      static_cast<const X*>(product), ld, logits, state, out, cu_q, state_slots, H, D, E, q_scale, tau))
+  DISTIE_DISPATCH(dtype, X, {                                                                                         \
+    if (logits != nullptr)                                                                                            \
+      gated_decay_scan_kernel<X, PARTS, ROWS, false><<<grid, 64 * PARTS, 0, stream>>>(                                \
+          static_cast<const X*>(product), ld, logits, nullptr, 0, nullptr, nullptr, 0, state, out, cu_q, state_slots, \
+          H, D, E, q_scale, tau);                                                                                     \
+    else                                                                                                              \
+      gated_decay_scan_kernel<X, PARTS, ROWS, true><<<grid, 64 * PARTS, 0, stream>>>(                                 \
+          static_cast<const X*>(product), ld, nullptr, static_cast<const X*>(low), ld_low, up, up_bias, rank, state,  \
+          out, cu_q, state_slots, H, D, E, q_scale, tau);                                                             \
+  })
   if (D <= 32) {
     DISTIE_GSCAN(4, 8);
   } else if (D <= 64) {

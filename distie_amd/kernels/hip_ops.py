@@ -312,7 +312,7 @@ class HipOps(Ops):
         o.distie_sigmoid_gate.argtypes = [_P, _I, _I, _I, _P, _I, _L, _P, _I, _I, _I, _P]
         o.distie_rmsnorm_gate.argtypes = [_P, _P, _I, _F, _P, _I, _L, _P, _I, _I, _I, _I, _I, _P]
         o.distie_norm_chain.argtypes = [_P, _I, _I, _P, _P, _I, _I, _P, _F, _F, _P, _F, _P, _P, _F, _P, _I, _P, _I, _I, _P]
-        o.distie_gated_decay_scan.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _P]
+        o.distie_gated_decay_scan.argtypes = [_P, _I, _L, _P, _P, _L, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _P]
         o.distie_gated_decay_scan_chunked.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P]
         o.distie_lru_gates.argtypes = [_P, _I, _L, _P, _P, _P, _P, _I, _P, _F, _P, _P, _I, _I, _I, _P]
         o.distie_lru_scan.argtypes = [_P, _P, _P, _P, _I, _L, _I, _P, _I, _P, _P, _I, _I, _P]
@@ -1329,19 +1329,38 @@ class HipOps(Ops):
             return self._norm_chain(delta.terms, delta.weights, delta.eps, delta.scale, post, residual, pre, out_dtype)
         return self._norm_chain([delta], None, 0.0, 1.0, post, residual, pre, out_dtype)
 
-    def gated_decay_scan(self, product, decay_logits, state, meta, num_heads, dim, value_dim, q_scale, tau):
+    def gated_decay_scan(self, product, decay_logits, state, meta, num_heads, dim, value_dim, q_scale, tau, decay_low=None):
         product = self.dense(product)
         self._own(product, decay_logits, state)
         T, W = product.shape
         if T != meta.num_tokens or W < num_heads * (2 * dim + value_dim):
             raise KernelError("gated_decay_scan: the product does not match the batch or the head counts")
-        if decay_logits.dtype != torch.float32 or tuple(decay_logits.shape) != (T, num_heads * dim):
-            raise KernelError("gated_decay_scan: the decay's logits are float32 [T, heads * dim]")
         if state.dtype != torch.float32 or tuple(state.shape[1:]) != (num_heads, dim, value_dim):
             raise KernelError("gated_decay_scan: the state is float32 [slots, heads, dim, value_dim]")
+        chunked = not self.captured and meta.host_cu_q is not None and meta.max_q >= self.SCAN_CHUNKED_MIN_ROWS and \
+            dim % 4 == 0 and value_dim % 4 == 0 and dim <= self._ops.distie_gated_decay_scan_chunked_max_dim()
+        low_ptr, low_ld, up, up_bias, rank = None, 0, None, None, 0
+        if decay_logits is None:
+            if decay_low is None:
+                raise KernelError("gated_decay_scan: neither the decay's logits nor what they are made from")
+            low, up, up_bias = decay_low
+            rank = up.shape[1]
+            if tuple(up.shape) != (num_heads * dim, rank) or low.shape[0] != T or low.dtype != product.dtype or \
+                    up_bias.dtype != torch.float32 or tuple(up_bias.shape) != (num_heads * dim,):
+                raise KernelError("gated_decay_scan: low [T, rank] of the product's dtype, up [heads * dim, rank], "
+                                  "bias float32 [heads * dim]")
+            if chunked or rank > self._ops.distie_gated_decay_scan_max_rank():
+                # portions of prompts (and wide projections): the logits as a product of their own
+                decay_logits = self.decay_logits_of(decay_low)
+            else:
+                low_ptr, low_ld = self._rows_view(low, rank)
+                up = self._f32(up)
+                self._own(up, up_bias)
+        if decay_logits is not None and (decay_logits.dtype != torch.float32 or
+                                         tuple(decay_logits.shape) != (T, num_heads * dim)):
+            raise KernelError("gated_decay_scan: the decay's logits are float32 [T, heads * dim]")
         out = torch.empty((T, num_heads * value_dim), dtype=torch.float32, device=self.device)
-        if not self.captured and meta.host_cu_q is not None and meta.max_q >= self.SCAN_CHUNKED_MIN_ROWS and \
-                dim % 4 == 0 and value_dim % 4 == 0 and dim <= self._ops.distie_gated_decay_scan_chunked_max_dim():
+        if chunked:
             # portions of prompts: chunks of rows side by side instead of one row after the other
             count, packed, scratch = self._scan_chunks(meta, self._ops.distie_gated_decay_scan_chunk_rows(), num_heads,
                                                        dim, value_dim)
@@ -1354,9 +1373,11 @@ class HipOps(Ops):
             _mark_written(state)
             return out
         _check(self._ops.distie_gated_decay_scan(
-            product.data_ptr(), _code(product), W, decay_logits.data_ptr(), state.data_ptr(), out.data_ptr(),
-            meta.cu_q.data_ptr(), meta.state_slots.data_ptr(), meta.num_requests, num_heads, dim, value_dim,
-            float(q_scale), float(tau), self._stream()), "gated_decay_scan")
+            product.data_ptr(), _code(product), W, decay_logits.data_ptr() if decay_logits is not None else None,
+            low_ptr, low_ld, up.data_ptr() if low_ptr is not None else None,
+            up_bias.data_ptr() if low_ptr is not None else None, rank if low_ptr is not None else 0, state.data_ptr(),
+            out.data_ptr(), meta.cu_q.data_ptr(), meta.state_slots.data_ptr(), meta.num_requests, num_heads, dim,
+            value_dim, float(q_scale), float(tau), self._stream()), "gated_decay_scan")
         _mark_written(state)
         return out
 

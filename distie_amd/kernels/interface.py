@@ -274,15 +274,24 @@ class Ops(abc.ABC):
         self.add_normed(residual, delta, post_weight, post_eps)
         return self.rmsnorm(residual, weight, eps, out_dtype)
 
-    def gated_decay_scan(self, product: torch.Tensor, decay_logits: torch.Tensor, state: torch.Tensor, meta: BatchMeta,
-                         num_heads: int, dim: int, value_dim: int, q_scale: float, tau: float) -> torch.Tensor:
+    def gated_decay_scan(self, product: torch.Tensor, decay_logits: Optional[torch.Tensor], state: torch.Tensor,
+                         meta: BatchMeta, num_heads: int, dim: int, value_dim: int, q_scale: float, tau: float,
+                         decay_low=None) -> torch.Tensor:
         """Linear attention whose state decays by a factor of its own for every key channel and token: with q
         (num_heads x dim, times `q_scale`), k (num_heads x dim) and v (num_heads x value_dim) from the first columns
         of `product` (act [T, W]) and alpha = sigmoid(decay_logits)^(1 / tau) (decay_logits float32 [T, num_heads *
         dim]), per head S <- diag(alpha) S + k v^T (alpha scales the rows of S, one a key channel) and o = S^T q.
         `state` float32 [slots + 1, num_heads, dim, value_dim] (rows by `meta.state_slots`) is read and left as
-        the step's last row leaves it. -> float32 [T, num_heads * value_dim]; decay, state and sums in float32."""
+        the step's last row leaves it. -> float32 [T, num_heads * value_dim]; decay, state and sums in float32.
+        `decay_logits` None: they are still to be made from `decay_low` = (low act [T, rank] or a view of columns, up
+        [num_heads * dim, rank], bias float32 [num_heads * dim]) as up . low + bias, float32 and not rounded; an
+        implementation may make them inside the scan (`decay_logits_of` makes them as a product of their own)."""
         raise NotImplementedError(f"{type(self).__name__} has no gated decayed state")
+
+    def decay_logits_of(self, decay_low) -> torch.Tensor:
+        """The decay's logits as a product of their own: float32 [T, num_heads * dim]."""
+        low, up, bias = decay_low
+        return self.linear_f32out(low.contiguous(), up, bias)
 
     def lru_gates(self, u: torch.Tensor, recur_weight: torch.Tensor, recur_bias: torch.Tensor,
                   input_weight: torch.Tensor, input_bias: torch.Tensor, lam: torch.Tensor, rate: float):

@@ -74,7 +74,9 @@ class GatedLinearAttention(Mixer):
     Every head's o goes through an RMS norm over its value_dim columns (weight `norm` [value_dim], the same for all
     heads), the heads side by side are multiplied by silu(W_g h) and projected by W_o. The state starts at zero and
     is float32 [heads, dim, value_dim] for each request; the decay (sigmoid, logarithm, power), the products k v^T
-    and S^T q and the norm are float32 in either precision; z is not rounded on its way into the recurrence."""
+    and S^T q and the norm are float32 in either precision; z is not rounded on its way into the recurrence. q, k, v,
+    the gate and W_a1 are one matrix product (their weights are stacked at load); z is made from its last columns,
+    inside the scan for steps of few rows."""
 
     def __init__(self, spec: PartSpec) -> None:
         super().__init__(spec)
@@ -89,7 +91,7 @@ class GatedLinearAttention(Mixer):
         if not self.tau > 0:
             raise ValueError("tau must be positive")
         self.q_scale = float(p.get("q_scale", self.head_dim ** -0.5))
-        self.in_weight = self.low_weight = self.up_weight = self.up_bias = self.out_weight = self.norm_weight = None
+        self.in_weight = self.up_weight = self.up_bias = self.out_weight = self.norm_weight = None
 
     def cache_requirement(self):
         return FixedState.of((self.num_heads, self.head_dim, self.value_dim))
@@ -105,8 +107,9 @@ class GatedLinearAttention(Mixer):
     def load(self, tensors) -> None:
         stacked = [tensors[name] for name in "qkvg"]
         dtype = torch.float32 if any(t.dtype == torch.float32 for t in stacked) else stacked[0].dtype
+        stacked.append(tensors["a1"])
+        dtype = torch.float32 if any(t.dtype == torch.float32 for t in stacked) else stacked[0].dtype
         self.in_weight = torch.cat([t.to(dtype) for t in stacked], dim=0).contiguous()
-        self.low_weight = tensors["a1"].contiguous()
         self.up_weight = tensors["a2"].contiguous()
         self.up_bias = tensors["a2.b"].float().contiguous()
         self.out_weight = tensors["o"].contiguous()
@@ -118,12 +121,12 @@ class GatedLinearAttention(Mixer):
 
     def forward(self, ops, x, ctx, cache, writes_cache: bool):
         product = ops.dense(ops.linear(x, self.in_weight))
-        low = ops.dense(ops.linear(x, self.low_weight))
-        logits = ops.linear_f32out(low, self.up_weight, self.up_bias)
-        mixed = ops.gated_decay_scan(product, logits, cache["state"], ctx.meta, self.num_heads, self.head_dim,
-                                     self.value_dim, self.q_scale, self.tau)
         first = self.num_heads * (2 * self.head_dim + self.value_dim)
-        gates = product[:, first:first + self.num_heads * self.value_dim]
+        behind = first + self.num_heads * self.value_dim
+        low = product[:, behind:behind + self.decay_rank]
+        mixed = ops.gated_decay_scan(product, None, cache["state"], ctx.meta, self.num_heads, self.head_dim,
+                                     self.value_dim, self.q_scale, self.tau, (low, self.up_weight, self.up_bias))
+        gates = product[:, first:behind]
         normed = ops.rmsnorm_gate(mixed, self.norm_weight, self.eps, gates, ctx.act_dtype, group=self.value_dim,
                                   gate="silu")
         return ops.linear(normed, self.out_weight)

@@ -120,25 +120,36 @@ def test_norms_behind_sub_layers_and_normed_sums(ops, width):
 @pytest.mark.parametrize("heads,dim,vdim,tau", [(2, 8, 16, 4.0), (3, 16, 8, 1.0), (1, 32, 32, 16.0), (2, 40, 72, 64.0),
                                                 (2, 128, 64, 16.0), (1, 12, 20, 2.0)])
 def test_gated_decayed_state(ops, heads, dim, vdim, tau, lengths, cuts):
-    """The state with a decay for every key channel and token, handed from step to step; decays from fast to slow."""
-    width = heads * (2 * dim + vdim) + 8                       # further columns are left alone
+    """The state with a decay for every key channel and token, handed from step to step; decays from fast to slow.
+    The decay's logits are given, or made from a few columns behind q, k and v (inside the scan, for few rows)."""
+    rank = 5 if dim == 12 else 8
+    first = heads * (2 * dim + vdim)
+    width = first + 3 + rank                                   # further columns are left alone; the last are `low`
+    up, bias = rnd(heads * dim, rank, seed=3, scale=1.5), rnd(heads * dim, seed=4, scale=2.0) + 2.0
     for dtype in act_types(ops):
         seqs = [rnd(n, width, seed=20 + i).to(dtype) for i, n in enumerate(lengths)]
-        logits = [rnd(n, heads * dim, seed=40 + i, scale=3.0) + 2.0 for i, n in enumerate(lengths)]
+        logits = [s[:, first + 3:].to(F) @ up.to(dtype).to(F).T + bias.to(F) for s in seqs]
         want = []
         for s, z in zip(seqs, logits):
             s = s.to(F)
             q = s[:, :heads * dim].view(-1, heads, dim) * dim ** -0.5
             k = s[:, heads * dim:2 * heads * dim].view(-1, heads, dim)
-            v = s[:, 2 * heads * dim:heads * (2 * dim + vdim)].view(-1, heads, vdim)
-            alpha = torch.sigmoid(z.to(F)).pow(1.0 / tau).view(-1, heads, dim)
+            v = s[:, 2 * heads * dim:first].view(-1, heads, vdim)
+            alpha = torch.sigmoid(z).pow(1.0 / tau).view(-1, heads, dim)
             want.append(plain.gated_linear_recurrence(q, k, v, alpha).reshape(-1, heads * vdim))
-        steps = Steps(ops, FixedState.of((heads, dim, vdim)), lengths, cuts)
-        for meta, rows in steps:
-            got = ops.gated_decay_scan(gather(seqs, rows).to(ops.device), gather(logits, rows).to(ops.device),
-                                       steps.view()["state"], meta, heads, dim, vdim, dim ** -0.5, tau)
-            assert got.dtype == torch.float32
-            close(got, gather(want, rows), torch.float32, f"rows {rows}")
+        for given in (True, False):
+            steps = Steps(ops, FixedState.of((heads, dim, vdim)), lengths, cuts)
+            for meta, rows in steps:
+                product = gather(seqs, rows).to(ops.device)
+                if given:
+                    got = ops.gated_decay_scan(product, gather(logits, rows).float().to(ops.device), steps.view()["state"],
+                                               meta, heads, dim, vdim, dim ** -0.5, tau)
+                else:
+                    low = (product[:, first + 3:], up.to(dtype).to(ops.device), bias.to(ops.device))
+                    got = ops.gated_decay_scan(product, None, steps.view()["state"], meta, heads, dim, vdim, dim ** -0.5,
+                                               tau, low)
+                assert got.dtype == torch.float32
+                close(got, gather(want, rows), torch.float32, f"rows {rows}, logits given: {given}")
 
 
 def test_norm_of_every_head_with_a_silu_gate(ops):

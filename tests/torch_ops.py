@@ -215,8 +215,10 @@ class TorchOps(Ops):
     def add_normed(self, residual, delta, weight, eps):
         residual += self._rms(delta, weight, eps)
 
-    def gated_decay_scan(self, product, decay_logits, state, meta, num_heads, dim, value_dim, q_scale, tau):
+    def gated_decay_scan(self, product, decay_logits, state, meta, num_heads, dim, value_dim, q_scale, tau, decay_low=None):
         T = product.shape[0]
+        if decay_logits is None:
+            decay_logits = self.decay_logits_of(decay_low)
         H, D, E = num_heads, dim, value_dim
         q = product[:, :H * D].float().view(T, H, D) * q_scale
         k = product[:, H * D:2 * H * D].float().view(T, H, D)
